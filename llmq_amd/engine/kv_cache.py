@@ -116,7 +116,9 @@ def blocks_needed(num_tokens: int, block_size: int) -> int:
 
 class RecurrentStateCache:
     """Per-sequence recurrent state, one fp32 tensor [num_slots + 1, *shape]
-    per recurrent layer (None for the others). A sequence owns one slot id
+    per recurrent layer (None for the others). A layer that carries several
+    states (a scan's state and the tail of its short convolution, say) names
+    a list of shapes and gets a list of tensors. A sequence owns one slot id
     across all layers from admission to release; slot ``num_slots`` is a
     scratch row for the padding rows of a captured decode graph. Slots are
     never cleared: a sequence's first portion starts from zero by itself."""
@@ -126,18 +128,29 @@ class RecurrentStateCache:
         self.layout = list(layout)
         self.num_slots = num_slots
         self.pad_slot = num_slots
+
+        def make(shape):
+            return torch.zeros(num_slots + 1, *shape, device=device, dtype=torch.float32)
+
         self.state: List[Optional[torch.Tensor]] = [
-            None if shape is None
-            else torch.zeros(num_slots + 1, *shape, device=device, dtype=torch.float32)
-            for shape in self.layout
+            None if entry is None
+            else [make(shape) for shape in entry] if isinstance(entry, list)
+            else make(entry)
+            for entry in self.layout
         ]
+
+    def _tensors(self):
+        for s in self.state:
+            if s is None:
+                continue
+            yield from (s if isinstance(s, list) else [s])
 
     @property
     def active(self) -> bool:
-        return any(s is not None for s in self.state)
+        return any(True for _ in self._tensors())
 
     def bytes(self) -> int:
-        return sum(s.numel() * 4 for s in self.state if s is not None)
+        return sum(t.numel() * 4 for t in self._tensors())
 
 
 class SlotAllocator:

@@ -612,12 +612,222 @@ KOSALORN_PRESETS = {
 }
 
 
+# ---------------------------------------------------------------------------
+# Muvetar: a hybrid decoder on an fp32 residual whose layers carry either a
+# minGRU recurrence or two mixers side by side (softmax attention with a
+# logarithmic distance penalty, and a Mamba selective scan), a mixture-of-
+# experts feed-forward with a shared expert, and a learned average over the
+# outputs of all earlier layers ("depth average") at every layer's end.
+# Positions enter through a sinusoidal vector added to the embedding and
+# through the attention's distance penalty only.
+
+
+@dataclass
+class MinGRUSpec:
+    """Gated recurrence whose gates read only the current token:
+    S_t = (1 - z_t) S_{t-1} + z_t c_t with z = sigmoid(.), c = g(.),
+    g(u) = u + 1/2 for u >= 0 and sigmoid(u) below; the output is
+    W_o (S_t * silu(W_g h))."""
+
+    width: int
+    kind: str = "mingru"
+
+
+@dataclass
+class LogBiasAttnSpec:
+    """Causal softmax attention with grouped key/value heads and no rotation;
+    head a's score for distance d = i - j is q.k * scale - r1_a ln(1 + r2_a d)."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    kind: str = "log_bias_attention"
+
+
+@dataclass
+class MambaSpec:
+    """Selective scan: a short causal convolution per channel, then per
+    channel c and state n  S <- exp(dt_c A[c, n]) S + dt_c x_c B_n,
+    y_c = sum_n S C_n + D_c x_c, gated by silu(z)."""
+
+    inner: int
+    state: int
+    dt_rank: int
+    conv: int
+    kind: str = "mamba"
+
+
+@dataclass
+class ParallelMixerSpec:
+    """Two mixers reading the same input; their outputs are added with fixed
+    scales."""
+
+    left: LogBiasAttnSpec
+    right: MambaSpec
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    kind: str = "parallel"
+
+
+@dataclass
+class SoftmaxMoESpec:
+    """Mixture of clamped gated experts: scores = softmax of the router
+    logits over ALL experts, the `top` largest chosen, their scores times
+    `scale` (not renormalised) weight the experts' OUTPUTS. Expert:
+    g = min(W_gate h, limit), u = clamp(W_up h, +-limit),
+    W_down(g * sigmoid(1.702 g) * (u + 1)). shared_ff > 0: one more expert of
+    the same form (own inner size and limit) runs for every token."""
+
+    experts: int
+    top: int
+    ff: int
+    limit: float
+    scale: float = 1.0
+    shared_ff: int = 0
+    shared_limit: float = 0.0
+
+
+@dataclass
+class MuvetarLayerSpec:
+    mixer: object                          # MinGRUSpec | ParallelMixerSpec
+    moe: Optional[SoftmaxMoESpec] = None   # None: the layer has no feed-forward
+
+
+@dataclass
+class MuvetarSpec:
+    name: str
+    family: str                   # "muvetar"
+    vocab_size: int
+    hidden_size: int
+    layers: list = field(default_factory=list)
+    rms_eps: float = 1e-6
+    residual_mult: float = 1.0    # every sublayer output is scaled by this
+    logit_softcap: float = 0.0    # 0 = none
+    max_position_embeddings: int = 1 << 17
+    tied_embeddings: bool = False
+    eos_token_id: int = 2
+    bos_token_id: int = 1
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def param_count(self) -> int:
+        w = self.hidden_size
+        total = 2 * self.vocab_size * w + w
+        for i, ls in enumerate(self.layers):
+            m = ls.mixer
+            total += w + (i + 2)
+            if m.kind == "mingru":
+                total += 3 * m.width * w + 2 * m.width + w * m.width
+            else:
+                a, r = m.left, m.right
+                total += (a.heads * a.dim + a.kv_heads * (a.dim + a.vdim)) * w
+                total += 2 * a.heads + w * a.heads * a.vdim
+                total += 2 * r.inner * w + r.inner * (r.conv + 1)
+                total += (r.dt_rank + 2 * r.state) * r.inner + r.inner * (r.dt_rank + 1)
+                total += r.inner * r.state + r.inner + w * r.inner
+            if ls.moe:
+                e = ls.moe
+                total += w + e.experts * (3 * w * e.ff + w) + 3 * w * e.shared_ff
+        return total
+
+
+def muvetar_spec_from_config(cfg: dict, name: str) -> MuvetarSpec:
+    """Muvetar config.json -> MuvetarSpec: every size and constant comes from
+    the config."""
+    layers = []
+    for i, lc in enumerate(cfg["layers"]):
+        mc, kind = lc["mixer"], lc["type"]
+        if kind == "mingru":
+            mixer = MinGRUSpec(width=int(mc["width"]))
+        elif kind == "parallel":
+            lt, rt = mc["left"], mc["right"]
+            heads = int(lt["heads"])
+            left = LogBiasAttnSpec(
+                heads=heads, kv_heads=int(lt.get("kv_heads", heads)), dim=int(lt["dim"]),
+                vdim=int(lt.get("vdim", lt["dim"])), scale=float(lt["scale"]))
+            if left.heads % left.kv_heads:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+            right = MambaSpec(inner=int(rt["inner"]), state=int(rt["state"]),
+                              dt_rank=int(rt["dt_rank"]), conv=int(rt["conv"]))
+            if right.conv < 1:
+                raise ValueError(f"layer {i}: the convolution needs at least one tap")
+            mixer = ParallelMixerSpec(left=left, right=right,
+                                      left_scale=float(mc.get("left_scale", 1.0)),
+                                      right_scale=float(mc.get("right_scale", 1.0)))
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        mlp, moe = lc.get("mlp"), None
+        if mlp is not None:
+            if mlp.get("kind", "moe") != "moe":
+                raise ValueError(f"layer {i}: unknown feed-forward kind {mlp.get('kind')!r}")
+            rt, ex, sh = mlp["router"], mlp["expert"], mlp.get("shared")
+            moe = SoftmaxMoESpec(
+                experts=int(rt["experts"]), top=int(rt["top"]), ff=int(ex["ff"]),
+                limit=float(ex["limit"]), scale=float(rt.get("scale", 1.0)),
+                shared_ff=int(sh["ff"]) if sh else 0,
+                shared_limit=float(sh["limit"]) if sh else 0.0)
+            if not 1 <= moe.top <= moe.experts:
+                raise ValueError(f"layer {i}: top must be within 1..experts")
+        layers.append(MuvetarLayerSpec(mixer=mixer, moe=moe))
+    return MuvetarSpec(
+        name=name, family="muvetar", vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]), layers=layers, rms_eps=float(cfg["norm"]["eps"]),
+        residual_mult=float(cfg.get("residual_mult", 1.0)),
+        logit_softcap=float(cfg.get("logit_softcap") or 0.0),
+    )
+
+
+def _muvetar(name, vocab, width, n_layers, heads, kv_heads, dim, vdim, inner, state, dt_rank,
+             experts, top, ff, shared_ff, parallel_every=2, gru_width=None, conv=4,
+             left_scale=1.0, right_scale=1.0, limit=7.0, router_scale=1.0, **kw):
+    """Preset builder: every `parallel_every`-th layer (starting with the
+    first) carries attention beside a selective scan, the others a minGRU;
+    every layer has the expert mixture with a shared expert."""
+    layers = []
+    for i in range(n_layers):
+        if i % parallel_every == 0:
+            mixer = ParallelMixerSpec(
+                LogBiasAttnSpec(heads, kv_heads, dim, vdim, dim ** -0.5),
+                MambaSpec(inner, state, dt_rank, conv), left_scale, right_scale)
+        else:
+            mixer = MinGRUSpec(gru_width or width)
+        layers.append(MuvetarLayerSpec(mixer, SoftmaxMoESpec(
+            experts, top, ff, limit, router_scale, shared_ff, limit)))
+    return MuvetarSpec(name=name, family="muvetar", vocab_size=vocab, hidden_size=width,
+                       layers=layers, **kw)
+
+
+MUVETAR_PRESETS = {
+    # CPU/GPU test config: both layer types, grouped kv heads, q/k size != v
+    # size, a recurrence narrower than the model, a state size that is no
+    # power of two
+    "tiny-muvetar": _muvetar("tiny-muvetar", 512, 64, 4, 4, 2, 16, 24, 96, 12, 6, 6, 2, 32, 48,
+                             gru_width=48, conv=3, left_scale=1.1, right_scale=0.8,
+                             limit=1.5, router_scale=1.3, residual_mult=0.5,
+                             logit_softcap=20.0),
+    # benchmark configs at the layer sizes of llama-3.2-1b / -3b and of the
+    # Kosalorn expert-mixture preset: same width, head count and depth; the
+    # scan is two model widths wide with 16 states per channel; 8 experts,
+    # 2 per token, each a quarter of the dense inner size, plus a shared one
+    "muvetar-1b": _muvetar("muvetar-1b", 128256, 2048, 16, 32, 8, 64, 64, 4096, 16, 128,
+                           8, 2, 2048, 2048),
+    "muvetar-3b": _muvetar("muvetar-3b", 128256, 3072, 28, 24, 8, 128, 128, 6144, 16, 192,
+                           8, 2, 2048, 2048),
+}
+
+
 def spec_from_hf_config(path: Path, name: str) -> ModelSpec:
     """Build a spec from a HF checkpoint directory's config.json."""
     with open(path / "config.json", "r", encoding="utf-8") as fh:
         cfg = json.load(fh)
     if str(cfg.get("architecture", "")).lower() == "kosalorn":
         return kosalorn_spec_from_config(cfg, name)
+    if str(cfg.get("architecture", "")).lower() == "muvetar":
+        return muvetar_spec_from_config(cfg, name)
     if str(cfg.get("architecture", "")).lower() == "kakovik":
         st = path / "model.safetensors"
         return kakovik_spec_from_config(
@@ -697,7 +907,9 @@ def resolve_spec(model: str) -> ModelSpec:
         return HYBRID_PRESETS[key]
     if key in KOSALORN_PRESETS:
         return KOSALORN_PRESETS[key]
+    if key in MUVETAR_PRESETS:
+        return MUVETAR_PRESETS[key]
     raise ValueError(
         f"Unknown model '{model}'. Provide a checkpoint directory with config.json "
-        f"or one of: {sorted(PRESETS) + sorted(HYBRID_PRESETS) + sorted(KOSALORN_PRESETS) + sorted(ALIASES)}"
+        f"or one of: {sorted(PRESETS) + sorted(HYBRID_PRESETS) + sorted(KOSALORN_PRESETS) + sorted(MUVETAR_PRESETS) + sorted(ALIASES)}"
     )

@@ -3,6 +3,7 @@
 from llmq_amd.engine.models.kakovik import KakovikLM
 from llmq_amd.engine.models.kosalorn import KosalornLM
 from llmq_amd.engine.models.llama import CausalLM
+from llmq_amd.engine.models.muvetar import MuvetarLM
 
 MODEL_CLASSES = {
     "llama": CausalLM,
@@ -11,6 +12,7 @@ MODEL_CLASSES = {
     "mistral": CausalLM,
     "kakovik": KakovikLM,
     "kosalorn": KosalornLM,
+    "muvetar": MuvetarLM,
 }
 
 
@@ -21,4 +23,4 @@ def model_class_for(spec):
         raise ValueError(f"no model class registered for family {spec.family!r}") from None
 
 
-__all__ = ["CausalLM", "KakovikLM", "KosalornLM", "MODEL_CLASSES", "model_class_for"]
+__all__ = ["CausalLM", "KakovikLM", "KosalornLM", "MuvetarLM", "MODEL_CLASSES", "model_class_for"]

@@ -259,4 +259,90 @@ def load_kosalorn_weights(model, path: Path) -> None:
     logger.info("loaded %d tensors from %s", len(tensors), path)
 
 
-_FAMILY_LOADERS = {"kakovik": load_kakovik_weights, "kosalorn": load_kosalorn_weights}
+def load_muvetar_weights(model, path: Path) -> None:
+    """Muvetar checkpoint names -> the packed in-tree tensors.
+
+    Checkpoint: 'embed', 'head', 'final.norm', and per layer 'l<i>.norm1',
+    'l<i>.norm2', 'l<i>.dwa', the mixer under 'l<i>.mix.' (a parallel layer's
+    two mixers under '.left.' and '.right.'), the feed-forward under
+    'l<i>.mlp.' (experts 'e<j>.', the shared expert 'shared.'); linear weights
+    are [out, in]. Packing: everything that reads the mixer's input -> 'in'
+    (segments at multiples of 8 rows), gate‖up -> one tensor, experts stacked
+    [E, ...], the attention's two distance numbers -> [heads, 2]."""
+    tensors = _read_all(path)
+    used = set()
+
+    def get(name: str) -> torch.Tensor:
+        if name not in tensors:
+            raise KeyError(f"missing tensor {name}")
+        used.add(name)
+        return tensors[name]
+
+    def copy_(dst: torch.Tensor, src: torch.Tensor) -> None:
+        if dst.shape != src.shape:
+            raise ValueError(f"shape mismatch: {tuple(dst.shape)} vs {tuple(src.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+    spec = model.spec
+    copy_(model.embedding, get("embed"))
+    copy_(model.lm_head, get("head"))
+    copy_(model.final_norm, get("final.norm"))
+    for i, (ls, lw) in enumerate(zip(spec.layers, model.layers)):
+        p, t, m = f"l{i}.", lw.t, ls.mixer
+        mx = p + "mix."
+        copy_(t["norm1"], get(p + "norm1"))
+        copy_(t["dwa"], get(p + "dwa"))
+
+        def put(seg: str, src: torch.Tensor, lw=lw, t=t) -> None:
+            at, n = lw.seg[seg]
+            copy_(t["in"][at:at + n], src)
+
+        t["in"].zero_()  # alignment rows between segments
+        if m.kind == "mingru":
+            put("z", get(mx + "z"))
+            put("u", get(mx + "x"))
+            put("g", get(mx + "g"))
+            copy_(t["z_b"], get(mx + "z.b"))
+            copy_(t["u_b"], get(mx + "x.b"))
+            copy_(t["o"], get(mx + "o"))
+        else:
+            lf, rt, r = mx + "left.", mx + "right.", m.right
+            put("q", get(lf + "q"))
+            put("k", get(lf + "k"))
+            put("v", get(lf + "v"))
+            copy_(t["r12"], torch.stack([get(lf + "r1").float(), get(lf + "r2").float()], dim=1))
+            copy_(t["attn_o"], get(lf + "o"))
+            w_in = get(rt + "in")
+            if w_in.shape[0] != 2 * r.inner:
+                raise ValueError(f"{rt}in: expected {2 * r.inner} rows")
+            put("x", w_in[: r.inner])
+            put("gate", w_in[r.inner:])
+            copy_(t["conv_w"], get(rt + "conv"))
+            copy_(t["conv_b"], get(rt + "conv.b"))
+            copy_(t["xproj"], get(rt + "x"))
+            copy_(t["dt"], get(rt + "dt"))
+            copy_(t["dt_b"], get(rt + "dt.b"))
+            copy_(t["A_log"], get(rt + "A_log"))
+            copy_(t["D"], get(rt + "D"))
+            copy_(t["scan_o"], get(rt + "o"))
+        if ls.moe:
+            e = ls.moe
+            copy_(t["norm2"], get(p + "norm2"))
+            copy_(t["router"], get(p + "mlp.router"))
+            for j in range(e.experts):
+                ep = f"{p}mlp.e{j}."
+                copy_(t["e_gate_up"][j], torch.cat([get(ep + "gate"), get(ep + "up")], dim=0))
+                copy_(t["e_down"][j], get(ep + "down"))
+            if e.shared_ff:
+                sp = p + "mlp.shared."
+                copy_(t["s_gate_up"], torch.cat([get(sp + "gate"), get(sp + "up")], dim=0))
+                copy_(t["s_down"], get(sp + "down"))
+    unused = sorted(set(tensors) - used)
+    if unused:
+        logger.warning("checkpoint tensors this configuration does not use: %s", unused[:8])
+    model.finalize()
+    logger.info("loaded %d tensors from %s", len(tensors), path)
+
+
+_FAMILY_LOADERS = {"kakovik": load_kakovik_weights, "kosalorn": load_kosalorn_weights,
+                   "muvetar": load_muvetar_weights}

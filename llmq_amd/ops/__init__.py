@@ -446,6 +446,9 @@ def qknorm_vmix_cache(q, k, v, q_w, k_w, v_first, lam: float, k_cache, v_cache,
 # positions (counted from 0), or the `span` newest positions up to the query
 _MASK_BLOCK, _MASK_WINDOW = 0, 1
 _NO_WINDOW = (1 << 31) - 1
+# bias modes: a table [H, n] indexed by the distance i - j, or per head the
+# pair (r1, r2) of a logarithmic distance penalty -r1 * ln(1 + r2 * (i - j))
+_BIAS_TABLE, _BIAS_LOG = 0, 1
 
 
 def chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables, cu_q, q_start,
@@ -455,7 +458,8 @@ def chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables, cu_q,
     if _use_hybrid(q):
         out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
         _HY.paged_attn_prefill(out, q, gate, k_cache, v_cache, bias, block_tables, cu_q,
-                               q_start, int(max_q), int(span), float(scale), _MASK_BLOCK, 1)
+                               q_start, int(max_q), int(span), float(scale), _MASK_BLOCK, 1,
+                               _BIAS_TABLE)
         return out
     return torch_ref.chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables,
                                              cu_q, q_start, span, scale)
@@ -467,7 +471,7 @@ def chunk_bias_attn_decode(q, gate, k_cache, v_cache, bias, block_tables, contex
     if _use_hybrid(q):
         out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
         _HY.paged_attn_decode(out, q, gate, k_cache, v_cache, bias, block_tables,
-                              context_lens, int(span), float(scale), _MASK_BLOCK)
+                              context_lens, int(span), float(scale), _MASK_BLOCK, _BIAS_TABLE)
         return out
     return torch_ref.chunk_bias_attn_decode(q, gate, k_cache, v_cache, bias, block_tables,
                                             context_lens, span, scale)
@@ -517,28 +521,31 @@ def head_norm(o, weight, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
 
 
 def window_attn_prefill(q, k_cache, v_cache, dv: int, block_tables, cu_q, q_start, max_q: int,
-                        window: int, scale: float) -> torch.Tensor:
+                        window: int, scale: float, log_bias=None) -> torch.Tensor:
     """Softmax attention of packed prompt portions over the paged cache:
     query at position i sees keys j <= i with i - j < window (window 0:
     every j <= i). v_cache None: the first dv channels of a key row are its
-    value (latent caches). q [T, H, D] -> [T, H, dv]."""
+    value (latent caches). log_bias fp32 [H, 2] = (r1, r2) per head: the
+    score loses r1 * ln(1 + r2 * (i - j)). q [T, H, D] -> [T, H, dv]."""
     if _use_hybrid(q):
         out = torch.empty(q.shape[0], q.shape[1], dv, dtype=q.dtype, device=q.device)
-        _HY.paged_attn_prefill(out, q, None, k_cache, v_cache, None, block_tables, cu_q, q_start,
-                               int(max_q), int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW, 1)
+        _HY.paged_attn_prefill(out, q, None, k_cache, v_cache, log_bias, block_tables, cu_q,
+                               q_start, int(max_q), int(window) or _NO_WINDOW, float(scale),
+                               _MASK_WINDOW, 1, _BIAS_LOG if log_bias is not None else _BIAS_TABLE)
         return out
     return torch_ref.window_attn_prefill(q, k_cache, v_cache, dv, block_tables, cu_q, q_start,
-                                         window, scale)
+                                         window, scale, log_bias)
 
 
 def window_attn_decode(q, k_cache, v_cache, dv: int, block_tables, context_lens, window: int,
-                       scale: float) -> torch.Tensor:
+                       scale: float, log_bias=None) -> torch.Tensor:
     """The single-token form: query b sits at position context_lens[b]-1."""
     if _use_hybrid(q):
         B, H, D = q.shape
         out = torch.empty(B, H, dv, dtype=q.dtype, device=q.device)
+        bias_mode = _BIAS_LOG if log_bias is not None else _BIAS_TABLE
         if (q.dtype == torch.bfloat16 and k_cache.shape[1] == 1 and H >= 8 and D % 8 == 0
-                and D <= 256 and q.is_contiguous()):
+                and D <= 256 and q.is_contiguous() and log_bias is None):
             # one kv head for all query heads: the heads of a token become the
             # rows of one head, all at the token's position, and the step runs
             # on the matrix-core kernel — every key tile staged once for all
@@ -546,13 +553,15 @@ def window_attn_decode(q, k_cache, v_cache, dv: int, block_tables, context_lens,
             cu = _head_row_offsets(B, H, q.device)
             _HY.paged_attn_prefill(out.view(B * H, 1, dv), q.view(B * H, 1, D), None, k_cache,
                                    v_cache, None, block_tables, cu, context_lens - 1, H,
-                                   int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW, 0)
+                                   int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW, 0,
+                                   _BIAS_TABLE)
             return out
-        _HY.paged_attn_decode(out, q, None, k_cache, v_cache, None, block_tables, context_lens,
-                              int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW)
+        _HY.paged_attn_decode(out, q, None, k_cache, v_cache, log_bias, block_tables,
+                              context_lens, int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW,
+                              bias_mode)
         return out
     return torch_ref.window_attn_decode(q, k_cache, v_cache, dv, block_tables, context_lens,
-                                        window, scale)
+                                        window, scale, log_bias)
 
 
 _HEAD_ROWS = {}
@@ -626,9 +635,13 @@ MOE_GROUP_MIN_ROWS = 16
 MOE_GROUP_MAX_ROWS = 2048
 
 
-def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False) -> torch.Tensor:
-    """Sum over a token's chosen experts of down_e(silu(gate_e x) * up_e x)
-    with x = w * h (the router score scales the expert's INPUT).
+def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False, act: str = "silu",
+                limit: float = 0.0, weight_output: bool = False) -> torch.Tensor:
+    """Sum over a token's chosen experts of down_e(act(gate_e x, up_e x)).
+    weight_output False: x = w * h (the router weight scales the expert's
+    INPUT); True: x = h and the weight scales the expert's OUTPUT.
+    act "silu": silu(g) * u; "clamp_swish": g * sigmoid(1.702 g) * (u + 1)
+    with g = min(g, limit), u = clamp(u, +-limit).
     h [T, W]; idx/w [T, top]; gate_up [E, 2F, W]; down [E, W, F].
 
     Few rows (or sync_free, for captured decode graphs): one matrix-vector
@@ -636,34 +649,152 @@ def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False) -> torch.Tens
     sorted by expert and one GEMM pair per expert on contiguous slices (the
     per-expert row counts cross to the host once)."""
     T, top = idx.shape
+    act_mode = _MOE_ACTS[act]
     if h.is_cuda and (sync_free or T * top <= MOE_GEMV_MAX_ROWS):
         _use_hybrid(h)
         F_ = down.shape[2]
         hmid = torch.empty(T * top, F_, dtype=h.dtype, device=h.device)
+        w_in = None if weight_output else w
         if MOE_GROUP_MIN_ROWS <= T * top <= MOE_GROUP_MAX_ROWS and \
                 max(h.shape[1], F_) * h.element_size() * 8 <= (128 << 10):
             # enough rows that experts repeat: grouped by expert inside the
             # kernel, a weight row is read once per 8 rows of its expert
-            _HY.moe_expert_gemv(hmid, h, idx, w, gate_up, True)
+            _HY.moe_expert_gemv(hmid, h, idx, w_in, gate_up, True, act_mode, float(limit))
             yk = torch.empty(T * top, h.shape[1], dtype=h.dtype, device=h.device)
-            _HY.moe_expert_gemv(yk, hmid, idx, None, down, False)
-            return yk.view(T, top, -1).float().sum(dim=1).to(h.dtype)
-        _HY.moe_gate_up_gemv(hmid, h, idx, w, gate_up)
+            _HY.moe_expert_gemv(yk, hmid, idx, None, down, False, 0, 0.0)
+            yk = yk.view(T, top, -1).float()
+            if weight_output:
+                yk = yk * w.unsqueeze(-1)
+            return yk.sum(dim=1).to(h.dtype)
+        _HY.moe_gate_up_gemv(hmid, h, idx, w_in, gate_up, act_mode, float(limit))
         y = torch.empty_like(h)
-        _HY.moe_down_gemv(y, hmid, idx, down)
+        _HY.moe_down_gemv(y, hmid, idx, down, w if weight_output else None)
         return y
     E = gate_up.shape[0]
     flat = idx.reshape(-1).long()
     order = torch.sort(flat, stable=True).indices
     counts = torch.bincount(flat, minlength=E).tolist()
-    xs = (h.float()[order // top] * w.reshape(-1)[order].unsqueeze(1)).to(h.dtype)
+    if weight_output:
+        xs = h[order // top]
+    else:
+        xs = (h.float()[order // top] * w.reshape(-1)[order].unsqueeze(1)).to(h.dtype)
     ys = torch.empty_like(xs)
     at = 0
     for e, n in enumerate(counts):
         if n:
-            act = act_and_mul(torch.nn.functional.linear(xs[at:at + n], gate_up[e]))
-            ys[at:at + n] = torch.nn.functional.linear(act, down[e])
+            gu = torch.nn.functional.linear(xs[at:at + n], gate_up[e])
+            mid = act_and_mul(gu) if act == "silu" else clamp_swish_mul(gu, limit)
+            ys[at:at + n] = torch.nn.functional.linear(mid, down[e])
             at += n
     inv = torch.empty_like(order)
     inv[order] = torch.arange(order.numel(), device=order.device)
-    return ys[inv].view(T, top, -1).float().sum(dim=1).to(h.dtype)
+    yk = ys[inv].view(T, top, -1).float()
+    if weight_output:
+        yk = yk * w.unsqueeze(-1)
+    return yk.sum(dim=1).to(h.dtype)
+
+
+_MOE_ACTS = {"silu": 0, "clamp_swish": 1}
+
+
+# ---- scan hybrids: elementwise gated recurrences, selective scans beside
+# attention, softmax-routed clamped experts, a learned average over layers --
+
+
+def embed_sinusoid(embedding, ids, positions, inv_freq) -> torch.Tensor:
+    """fp32 [T, W]: embedding[ids] plus the sinusoidal position vector (entry
+    2i = sin(p * inv_freq[i]), entry 2i+1 = cos of it, angles in fp32)."""
+    if _use_hybrid(embedding):
+        out = torch.empty(ids.shape[0], embedding.shape[1], dtype=torch.float32,
+                          device=embedding.device)
+        _HY.embed_sinusoid(out, embedding, ids, positions, inv_freq)
+        return out
+    return torch_ref.embed_sinusoid(embedding, ids, positions, inv_freq)
+
+
+def scaled_add_norm(res, y, y2, a1: float, a2: float, weight, eps: float,
+                    out_dtype: torch.dtype) -> torch.Tensor:
+    """res (fp32, in place) += a1 * y [+ a2 * y2]; returns rmsnorm(res) * weight
+    in out_dtype."""
+    if _use_hybrid(res):
+        out = torch.empty(res.shape, dtype=out_dtype, device=res.device)
+        _HY.scaled_add_norm(out, res, y, y2, float(a1), float(a2), weight, float(eps))
+        return out
+    return torch_ref.scaled_add_norm(res, y, y2, a1, a2, weight, eps, out_dtype)
+
+
+def depth_mix_norm(stack, n: int, coef, y, y2, a1: float, a2: float, weight, eps: float,
+                   out_dtype: torch.dtype) -> torch.Tensor:
+    """The close of a layer under a learned average over layer outputs.
+    stack [>= n+1, T, W] fp32: rows 0..n-1 hold the embedding output and the
+    layer results so far. Row n-1 (in place) += a1 * y [+ a2 * y2]; row n =
+    sum_j coef[j] * row j; returns rmsnorm(row n) * weight in out_dtype."""
+    if _use_hybrid(stack):
+        out = torch.empty(stack.shape[1:], dtype=out_dtype, device=stack.device)
+        _HY.depth_mix_norm(out, stack, int(n), coef, y, y2, float(a1), float(a2), weight,
+                           float(eps))
+        return out
+    return torch_ref.depth_mix_norm(stack, n, coef, y, y2, a1, a2, weight, eps, out_dtype)
+
+
+def kv_scatter(k, v, k_cache, v_cache, slots) -> None:
+    """Rows of k [T, G*D] and v [T, G*DV] (column slices of a projection)
+    into the paged cache rows `slots`; a negative slot writes nothing."""
+    if _use_hybrid(k):
+        _HY.kv_scatter(k, v, k_cache, v_cache, slots)
+        return
+    torch_ref.kv_scatter(k, v, k_cache, v_cache, slots)
+
+
+def mingru_scan(z, u, g, z_b, u_b, state, cu, slots, fresh, out_dtype: torch.dtype):
+    """minGRU over packed sequences: S <- (1 - a) S + a c per channel with
+    a = sigmoid(z + z_b), c = u' + 1/2 (u' >= 0) else sigmoid(u'), u' = u +
+    u_b; state [slots, n] fp32 advanced in place; returns S_t * silu(g_t)."""
+    if _use_hybrid(z):
+        out = torch.empty(z.shape, dtype=out_dtype, device=z.device)
+        _HY.mingru_scan(out, z, u, g, z_b, u_b, state, cu, slots, fresh)
+        return out
+    return torch_ref.mingru_scan(z, u, g, z_b, u_b, state, cu, slots, fresh, out_dtype)
+
+
+def causal_conv_silu(x, weight, bias, tail, cu, slots, fresh) -> torch.Tensor:
+    """Per-channel causal convolution + SiLU over packed sequences; tail
+    [slots, K-1, C] fp32 carries each sequence's last K-1 inputs."""
+    if _use_hybrid(x):
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _HY.causal_conv_silu(out, x, weight, bias, tail, cu, slots, fresh)
+        return out
+    return torch_ref.causal_conv_silu(x, weight, bias, tail, cu, slots, fresh)
+
+
+def selective_scan(x, dt, dt_b, A, Bm, Cm, D, z, state, cu, slots, fresh) -> torch.Tensor:
+    """Selective scan over packed sequences (see torch_ref.selective_scan);
+    state [slots, C, N] fp32 advanced in place; returns y * silu(z)."""
+    if _use_hybrid(x):
+        out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
+        _HY.selective_scan(out, x, dt, dt_b, A, Bm, Cm, D, z, state, cu, slots, fresh)
+        return out
+    return torch_ref.selective_scan(x, dt, dt_b, A, Bm, Cm, D, z, state, cu, slots, fresh)
+
+
+def softmax_topk(logits, top: int, scale: float = 1.0):
+    """Router: softmax over all experts in fp32, the `top` largest per row,
+    times scale: (indices int32 [T, top], weights fp32 [T, top])."""
+    if _use_hybrid(logits):
+        T = logits.shape[0]
+        idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
+        w = torch.empty(T, top, dtype=torch.float32, device=logits.device)
+        _HY.softmax_topk(idx, w, logits, int(top), float(scale))
+        return idx, w
+    return torch_ref.softmax_topk(logits, top, scale)
+
+
+def clamp_swish_mul(x, limit: float) -> torch.Tensor:
+    """[*, 2d] -> g * sigmoid(1.702 g) * (u + 1), g = min(x[..., :d], limit),
+    u = clamp(x[..., d:], -limit, limit)."""
+    if _use_hybrid(x):
+        d = x.shape[-1] // 2
+        out = torch.empty(*x.shape[:-1], d, dtype=x.dtype, device=x.device)
+        _HY.clamp_swish_mul(out, x, float(limit))
+        return out
+    return torch_ref.clamp_swish_mul(x, limit)

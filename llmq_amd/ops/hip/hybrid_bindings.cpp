@@ -173,7 +173,7 @@ struct AttnDims { int H, G, D, DV, bs, v_row; const void* vptr; const float* bia
 AttnDims attn_check(const at::Tensor& out, const at::Tensor& q, const std::optional<at::Tensor>& gate,
                     const at::Tensor& k_cache, const std::optional<at::Tensor>& v_cache,
                     const std::optional<at::Tensor>& bias, const at::Tensor& block_tables,
-                    long span, long mask_mode) {
+                    long span, long mask_mode, long bias_mode) {
   HY_GPU(q);
   TORCH_CHECK(q.dim() == 3 && out.dim() == 3, "q [T, H, D], out [T, H, DV]");
   HY_INNER(q); HY_INNER(out);
@@ -198,10 +198,14 @@ AttnDims attn_check(const at::Tensor& out, const at::Tensor& q, const std::optio
   TORCH_CHECK(a.H % a.G == 0, "heads must be a multiple of kv heads");
   TORCH_CHECK(a.DV >= 1 && a.DV <= 512, "value size above 512 is not supported");
   TORCH_CHECK(span >= 1);
+  TORCH_CHECK(bias_mode == kBiasTable || bias_mode == kBiasLog, "unknown bias mode");
   if (bias.has_value()) {
     TORCH_CHECK(bias->scalar_type() == at::kFloat && bias->is_contiguous() && bias->dim() == 2 &&
-                bias->size(0) == a.H && bias->size(1) >= 1 && bias->size(1) <= span,
-                "bias must be fp32 [H, n], n = min(span, longest context the engine admits)");
+                bias->size(0) == a.H && bias->is_cuda(), "bias must be fp32 [H, n] on the GPU");
+    TORCH_CHECK(bias_mode == kBiasLog ? bias->size(1) == 2
+                                      : bias->size(1) >= 1 && bias->size(1) <= span,
+                "bias is [H, 2] = (r1, r2) per head in log mode, else [H, n] with "
+                "n = min(span, longest context the engine admits)");
     a.bias = bias->data_ptr<float>();
     a.bias_len = (int)bias->size(1);
   }
@@ -227,10 +231,11 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
                         at::Tensor k_cache, const std::optional<at::Tensor>& v_cache,
                         const std::optional<at::Tensor>& bias, at::Tensor block_tables,
                         at::Tensor cu_q, at::Tensor q_start, int64_t max_q, int64_t span,
-                        double scale, int64_t mask_mode, int64_t pos_stride) {
+                        double scale, int64_t mask_mode, int64_t pos_stride, int64_t bias_mode) {
   if (q.size(0) == 0) return;
   TORCH_CHECK(pos_stride == 0 || pos_stride == 1, "pos_stride is 0 (rows share a position) or 1");
-  const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span, mask_mode);
+  const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span, mask_mode,
+                                bias_mode);
   HY_I32(cu_q); HY_I32(q_start);
   const int B = q_start.numel();
   TORCH_CHECK(cu_q.numel() == B + 1 && block_tables.size(0) == B && max_q >= 1);
@@ -277,7 +282,7 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
                          (int)span, (float)scale, a.v_row, (int)mask_mode, (int)pos_stride,
-                         n_split, n_split > 1 ? part.data_ptr<float>() : nullptr);
+                         n_split, n_split > 1 ? part.data_ptr<float>() : nullptr, (int)bias_mode);
     };
     if (ksn <= 2 && dtn <= 4) launch.template operator()<2, 4>();
     else if (ksn <= 4 && dtn <= 8) launch.template operator()<4, 8>();
@@ -308,7 +313,7 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
                          reinterpret_cast<const T*>(a.vptr), a.bias, a.bias_len,
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
-                         (int)span, (float)scale, a.v_row, (int)mask_mode);
+                         (int)span, (float)scale, a.v_row, (int)mask_mode, (int)bias_mode);
     });
   });
 }
@@ -316,9 +321,11 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
 void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Tensor>& gate,
                        at::Tensor k_cache, const std::optional<at::Tensor>& v_cache,
                        const std::optional<at::Tensor>& bias, at::Tensor block_tables,
-                       at::Tensor context_lens, int64_t span, double scale, int64_t mask_mode) {
+                       at::Tensor context_lens, int64_t span, double scale, int64_t mask_mode,
+                       int64_t bias_mode) {
   if (q.size(0) == 0) return;
-  const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span, mask_mode);
+  const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span, mask_mode,
+                                bias_mode);
   HY_I32(context_lens);
   const int B = q.size(0);
   TORCH_CHECK(context_lens.numel() == B && block_tables.size(0) == B);
@@ -345,7 +352,7 @@ void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Ten
                          reinterpret_cast<const T*>(a.vptr), a.bias, a.bias_len,
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          context_lens.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs, (int)span,
-                         (float)scale, a.v_row, (int)mask_mode);
+                         (float)scale, a.v_row, (int)mask_mode, (int)bias_mode);
       };
       if (hpw == 8) launch.template operator()<8>();
       else if (hpw == 4) launch.template operator()<4>();
@@ -572,14 +579,22 @@ MoeDims moe_check(const at::Tensor& idx, int W, int F, int E) {
   return MoeDims{idx.size(0), (int)idx.size(1), W, F, E};
 }
 
-void moe_gate_up_gemv(at::Tensor hmid, at::Tensor h, at::Tensor idx, at::Tensor w, at::Tensor gate_up) {
+void moe_gate_up_gemv(at::Tensor hmid, at::Tensor h, at::Tensor idx,
+                      const std::optional<at::Tensor>& w, at::Tensor gate_up, int64_t act,
+                      double limit) {
   HY_GPU(h);
   TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && gate_up.dim() == 3 && gate_up.is_contiguous());
   TORCH_CHECK(gate_up.size(1) % 2 == 0 && gate_up.size(2) == h.size(1));
   const MoeDims m = moe_check(idx, h.size(1), gate_up.size(1) / 2, gate_up.size(0));
   if (m.T == 0) return;
   TORCH_CHECK(idx.size(0) == h.size(0));
-  TORCH_CHECK(w.scalar_type() == at::kFloat && w.is_contiguous() && w.sizes() == idx.sizes());
+  TORCH_CHECK(act == kMoeActSilu || act == kMoeActClampSwish, "unknown expert activation");
+  const float* wp = nullptr;
+  if (w.has_value()) {
+    TORCH_CHECK(w->scalar_type() == at::kFloat && w->is_contiguous() && w->sizes() == idx.sizes() &&
+                w->is_cuda());
+    wp = w->data_ptr<float>();
+  }
   TORCH_CHECK(hmid.is_contiguous() && hmid.dim() == 2 && hmid.size(0) == m.T * m.top && hmid.size(1) == m.F);
   TORCH_CHECK(hmid.scalar_type() == h.scalar_type() && gate_up.scalar_type() == h.scalar_type());
   const size_t lds = sizeof(float) * (size_t)m.W;
@@ -589,12 +604,13 @@ void moe_gate_up_gemv(at::Tensor hmid, at::Tensor h, at::Tensor idx, at::Tensor 
     allow_lds(kern, lds);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(), reinterpret_cast<T*>(hmid.data_ptr()),
                        reinterpret_cast<const T*>(h.data_ptr()), idx.data_ptr<int>(),
-                       w.data_ptr<float>(), reinterpret_cast<const T*>(gate_up.data_ptr()), m.top,
-                       m.W, m.F, m.E);
+                       wp, reinterpret_cast<const T*>(gate_up.data_ptr()), m.top,
+                       m.W, m.F, m.E, (int)act, (float)limit);
   });
 }
 
-void moe_down_gemv(at::Tensor y, at::Tensor hmid, at::Tensor idx, at::Tensor down) {
+void moe_down_gemv(at::Tensor y, at::Tensor hmid, at::Tensor idx, at::Tensor down,
+                   const std::optional<at::Tensor>& wo) {
   HY_GPU(hmid);
   TORCH_CHECK(down.dim() == 3 && down.is_contiguous() && hmid.dim() == 2 && hmid.is_contiguous());
   const MoeDims m = moe_check(idx, down.size(1), down.size(2), down.size(0));
@@ -602,6 +618,12 @@ void moe_down_gemv(at::Tensor y, at::Tensor hmid, at::Tensor idx, at::Tensor dow
   TORCH_CHECK(hmid.size(0) == m.T * m.top && hmid.size(1) == m.F);
   TORCH_CHECK(y.is_contiguous() && y.dim() == 2 && y.size(0) == m.T && y.size(1) == m.W);
   TORCH_CHECK(y.scalar_type() == hmid.scalar_type() && down.scalar_type() == hmid.scalar_type());
+  const float* wop = nullptr;
+  if (wo.has_value()) {
+    TORCH_CHECK(wo->scalar_type() == at::kFloat && wo->is_contiguous() && wo->sizes() == idx.sizes() &&
+                wo->is_cuda());
+    wop = wo->data_ptr<float>();
+  }
   const size_t lds = sizeof(float) * (size_t)m.top * m.F;
   const dim3 grid((m.W + 4 * kMoeRowsPerWave - 1) / (4 * kMoeRowsPerWave), m.T);
   hy_dispatch(hmid, "moe_down_gemv", [&]<typename T>() {
@@ -609,15 +631,16 @@ void moe_down_gemv(at::Tensor y, at::Tensor hmid, at::Tensor idx, at::Tensor dow
     allow_lds(kern, lds);
     hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(), reinterpret_cast<T*>(y.data_ptr()),
                        reinterpret_cast<const T*>(hmid.data_ptr()), idx.data_ptr<int>(),
-                       reinterpret_cast<const T*>(down.data_ptr()), m.top, m.W, m.F, m.E);
+                       reinterpret_cast<const T*>(down.data_ptr()), m.top, m.W, m.F, m.E, wop);
   });
 }
 
 // Expert mixture grouped by expert, no host sync. gate_up: in = h [T, W],
 // out = hmid [T*top, F]; else: in = hmid [T*top, F], out = yk [T*top, W].
 void moe_expert_gemv(at::Tensor out, at::Tensor in, at::Tensor idx, const std::optional<at::Tensor>& w,
-                     at::Tensor weight, bool gate_up) {
+                     at::Tensor weight, bool gate_up, int64_t act, double limit) {
   HY_GPU(in);
+  TORCH_CHECK(act == kMoeActSilu || act == kMoeActClampSwish, "unknown expert activation");
   HY_I32(idx);
   TORCH_CHECK(idx.dim() == 2 && idx.size(1) >= 1, "idx must be [T, top]");
   const long rows = idx.numel();
@@ -632,9 +655,10 @@ void moe_expert_gemv(at::Tensor out, at::Tensor in, at::Tensor idx, const std::o
   TORCH_CHECK(in.size(0) == (gate_up ? idx.size(0) : rows));
   TORCH_CHECK(in.scalar_type() == out.scalar_type() && weight.scalar_type() == out.scalar_type());
   const float* wp = nullptr;
-  if (gate_up) {
-    TORCH_CHECK(weight.size(1) % 2 == 0 && w.has_value() && w->scalar_type() == at::kFloat &&
-                w->is_contiguous() && w->numel() == rows && w->is_cuda());
+  if (gate_up) TORCH_CHECK(weight.size(1) % 2 == 0);
+  if (gate_up && w.has_value()) {
+    TORCH_CHECK(w->scalar_type() == at::kFloat && w->is_contiguous() && w->numel() == rows &&
+                w->is_cuda());
     wp = w->data_ptr<float>();
   }
   const dim3 grid((N + 4 * kMoeFPW - 1) / (4 * kMoeFPW), E);
@@ -645,10 +669,313 @@ void moe_expert_gemv(at::Tensor out, at::Tensor in, at::Tensor idx, const std::o
       allow_lds(kern, lds);
       hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(), reinterpret_cast<T*>(out.data_ptr()),
                          reinterpret_cast<const T*>(in.data_ptr()), idx.data_ptr<int>(), wp,
-                         reinterpret_cast<const T*>(weight.data_ptr()), (int)rows, top, K, N);
+                         reinterpret_cast<const T*>(weight.data_ptr()), (int)rows, top, K, N,
+                         (int)act, (float)limit);
     };
     if (gate_up) launch.template operator()<true>();
     else launch.template operator()<false>();
+  });
+}
+
+
+// ---- scan/attention hybrids ------------------------------------------------
+
+#define HY_F32(x) TORCH_CHECK(x.scalar_type() == at::kFloat && x.is_contiguous() && x.is_cuda(), #x " must be contiguous fp32 on the GPU")
+
+void embed_sinusoid(at::Tensor out, at::Tensor embedding, at::Tensor ids, at::Tensor positions,
+                    at::Tensor inv_freq) {
+  HY_GPU(embedding);
+  TORCH_CHECK(embedding.dim() == 2 && embedding.is_contiguous());
+  const long rows = ids.numel();
+  const int W = embedding.size(1);
+  if (rows == 0) return;
+  TORCH_CHECK(ids.scalar_type() == at::kLong && ids.is_contiguous() && ids.is_cuda());
+  TORCH_CHECK(positions.scalar_type() == at::kLong && positions.is_contiguous() &&
+              positions.numel() == rows && positions.is_cuda());
+  HY_F32(inv_freq); HY_F32(out);
+  TORCH_CHECK(inv_freq.numel() == (W + 1) / 2, "inv_freq needs one entry per (sin, cos) pair");
+  TORCH_CHECK(out.dim() == 2 && out.size(0) == rows && out.size(1) == W);
+  hy_dispatch(embedding, "embed_sinusoid", [&]<typename T>() {
+    hipLaunchKernelGGL(embed_sinusoid_kernel<T>, dim3(rows), dim3(256), 0, hy_stream(),
+                       out.data_ptr<float>(), reinterpret_cast<const T*>(embedding.data_ptr()),
+                       ids.data_ptr<long>(), positions.data_ptr<long>(), inv_freq.data_ptr<float>(),
+                       W, (long)embedding.size(0));
+  });
+}
+
+void scaled_add_norm(at::Tensor out, at::Tensor res, at::Tensor y, const std::optional<at::Tensor>& y2,
+                     double a1, double a2, at::Tensor weight, double eps) {
+  HY_GPU(y);
+  HY_F32(res);
+  TORCH_CHECK(y.dim() == 2 && y.is_contiguous() && out.is_contiguous() && weight.is_contiguous());
+  const long rows = y.size(0);
+  const int W = y.size(1);
+  if (rows == 0) return;
+  TORCH_CHECK(res.sizes() == y.sizes() && out.sizes() == y.sizes() && weight.numel() == W);
+  TORCH_CHECK(out.scalar_type() == y.scalar_type() && weight.scalar_type() == y.scalar_type());
+  const void* y2p = nullptr;
+  if (y2.has_value()) {
+    TORCH_CHECK(y2->is_contiguous() && y2->sizes() == y.sizes() && y2->scalar_type() == y.scalar_type() &&
+                y2->is_cuda());
+    y2p = y2->data_ptr();
+  }
+  if (y.scalar_type() == at::kBFloat16 && W % 8 == 0 && W <= 4 * 2048) {
+    using bf = __hip_bfloat16;
+    auto launch = [&]<int CH>() {
+      hipLaunchKernelGGL(scaled_add_norm_vec_kernel<CH>, dim3(rows), dim3(256), 0, hy_stream(),
+                         reinterpret_cast<bf*>(out.data_ptr()), res.data_ptr<float>(),
+                         reinterpret_cast<const bf*>(y.data_ptr()), reinterpret_cast<const bf*>(y2p),
+                         (float)a1, (float)a2, reinterpret_cast<const bf*>(weight.data_ptr()), W,
+                         (float)eps);
+    };
+    if (W <= 2048) launch.template operator()<1>();
+    else if (W <= 4096) launch.template operator()<2>();
+    else launch.template operator()<4>();
+    return;
+  }
+  hy_dispatch(y, "scaled_add_norm", [&]<typename T>() {
+    hipLaunchKernelGGL(scaled_add_norm_kernel<T>, dim3(rows), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(out.data_ptr()), res.data_ptr<float>(),
+                       reinterpret_cast<const T*>(y.data_ptr()), reinterpret_cast<const T*>(y2p),
+                       (float)a1, (float)a2, reinterpret_cast<const T*>(weight.data_ptr()), W,
+                       (float)eps);
+  });
+}
+
+void depth_mix_norm(at::Tensor out, at::Tensor stack, int64_t n, at::Tensor coef, at::Tensor y,
+                    const std::optional<at::Tensor>& y2, double a1, double a2, at::Tensor weight,
+                    double eps) {
+  HY_GPU(y);
+  HY_F32(stack); HY_F32(coef);
+  TORCH_CHECK(y.dim() == 2 && y.is_contiguous() && out.is_contiguous() && weight.is_contiguous());
+  const long rows = y.size(0);
+  const int W = y.size(1);
+  if (rows == 0) return;
+  TORCH_CHECK(stack.dim() == 3 && stack.size(1) == rows && stack.size(2) == W);
+  TORCH_CHECK(n >= 1 && n + 1 <= stack.size(0) && coef.numel() >= n,
+              "the stack needs entries 0..n and one coefficient per entry below n");
+  TORCH_CHECK(out.sizes() == y.sizes() && weight.numel() == W);
+  TORCH_CHECK(out.scalar_type() == y.scalar_type() && weight.scalar_type() == y.scalar_type());
+  const void* y2p = nullptr;
+  if (y2.has_value()) {
+    TORCH_CHECK(y2->is_contiguous() && y2->sizes() == y.sizes() && y2->scalar_type() == y.scalar_type() &&
+                y2->is_cuda());
+    y2p = y2->data_ptr();
+  }
+  const long ls = rows * (long)W;
+  if (y.scalar_type() == at::kBFloat16 && W % 4 == 0 && W <= 8 * 1024) {
+    using bf = __hip_bfloat16;
+    auto launch = [&]<int CH>() {
+      hipLaunchKernelGGL(depth_mix_norm_vec_kernel<CH>, dim3(rows), dim3(256), 0, hy_stream(),
+                         reinterpret_cast<bf*>(out.data_ptr()), stack.data_ptr<float>(), ls, (int)n,
+                         coef.data_ptr<float>(), reinterpret_cast<const bf*>(y.data_ptr()),
+                         reinterpret_cast<const bf*>(y2p), (float)a1, (float)a2,
+                         reinterpret_cast<const bf*>(weight.data_ptr()), W, (float)eps);
+    };
+    if (W <= 1024) launch.template operator()<1>();
+    else if (W <= 2048) launch.template operator()<2>();
+    else if (W <= 4096) launch.template operator()<4>();
+    else launch.template operator()<8>();
+    return;
+  }
+  hy_dispatch(y, "depth_mix_norm", [&]<typename T>() {
+    hipLaunchKernelGGL(depth_mix_norm_kernel<T>, dim3(rows), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(out.data_ptr()), stack.data_ptr<float>(), ls, (int)n,
+                       coef.data_ptr<float>(), reinterpret_cast<const T*>(y.data_ptr()),
+                       reinterpret_cast<const T*>(y2p), (float)a1, (float)a2,
+                       reinterpret_cast<const T*>(weight.data_ptr()), W, (float)eps);
+  });
+}
+
+// k [T, G*D], v [T, G*DV]: row-strided views of one GEMM output.
+void kv_scatter(at::Tensor k, at::Tensor v, at::Tensor k_cache, at::Tensor v_cache, at::Tensor slots) {
+  HY_GPU(k);
+  HY_INNER(k); HY_INNER(v);
+  TORCH_CHECK(k.dim() == 2 && v.dim() == 2);
+  const long T_ = k.size(0);
+  if (T_ == 0) return;
+  TORCH_CHECK(v.size(0) == T_ && slots.numel() == T_);
+  TORCH_CHECK(slots.scalar_type() == at::kLong && slots.is_contiguous() && slots.is_cuda());
+  TORCH_CHECK(k_cache.dim() == 4 && v_cache.dim() == 4 && k_cache.is_contiguous() && v_cache.is_contiguous());
+  const int G = k_cache.size(1), bs = k_cache.size(2), D = k_cache.size(3), DV = v_cache.size(3);
+  TORCH_CHECK(v_cache.size(0) == k_cache.size(0) && v_cache.size(1) == G && v_cache.size(2) == bs);
+  TORCH_CHECK(k.size(1) == G * D && v.size(1) == G * DV, "k/v widths do not match the cache layout");
+  const auto dt = k.scalar_type();
+  TORCH_CHECK(v.scalar_type() == dt && k_cache.scalar_type() == dt && v_cache.scalar_type() == dt,
+              "kv_scatter: one dtype for activations and cache");
+  hy_dispatch(k, "kv_scatter", [&]<typename T>() {
+    hipLaunchKernelGGL(kv_scatter_kernel<T>, dim3(T_), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<const T*>(k.data_ptr()), k.stride(0),
+                       reinterpret_cast<const T*>(v.data_ptr()), v.stride(0),
+                       reinterpret_cast<T*>(k_cache.data_ptr()), reinterpret_cast<T*>(v_cache.data_ptr()),
+                       slots.data_ptr<long>(), G, D, DV, bs);
+  });
+}
+
+struct SeqDims { int B; };
+
+SeqDims seq_check(const at::Tensor& cu, const at::Tensor& slots, const at::Tensor& fresh,
+                  const at::Tensor& state) {
+  HY_I32(cu); HY_I32(slots); HY_I32(fresh);
+  TORCH_CHECK(cu.is_cuda() && slots.is_cuda() && fresh.is_cuda());
+  const int B = slots.numel();
+  TORCH_CHECK(cu.numel() == B + 1 && fresh.numel() == B);
+  TORCH_CHECK(state.scalar_type() == at::kFloat && state.is_contiguous() && state.is_cuda(),
+              "state must be contiguous fp32 on the GPU");
+  return SeqDims{B};
+}
+
+// z, u, g [T, n]: row-strided slices of one projection output (same stride).
+void mingru_scan(at::Tensor out, at::Tensor z, at::Tensor u, at::Tensor g, at::Tensor z_b,
+                 at::Tensor u_b, at::Tensor state, at::Tensor cu, at::Tensor slots, at::Tensor fresh) {
+  HY_GPU(z);
+  HY_INNER(z); HY_INNER(u); HY_INNER(g);
+  TORCH_CHECK(z.dim() == 2 && u.sizes() == z.sizes() && g.sizes() == z.sizes());
+  const long T_ = z.size(0);
+  const int n = z.size(1);
+  if (T_ == 0) return;
+  TORCH_CHECK(u.stride(0) == z.stride(0) && g.stride(0) == z.stride(0), "z, u, g must share a row stride");
+  TORCH_CHECK(u.scalar_type() == z.scalar_type() && g.scalar_type() == z.scalar_type() &&
+              out.scalar_type() == z.scalar_type());
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == z.sizes());
+  HY_F32(z_b); HY_F32(u_b);
+  TORCH_CHECK(z_b.numel() == n && u_b.numel() == n);
+  const SeqDims d = seq_check(cu, slots, fresh, state);
+  TORCH_CHECK(state.dim() == 2 && state.size(1) == n, "state [slots, n] fp32");
+  const dim3 grid((n + 255) / 256, d.B);
+  hy_dispatch(z, "mingru_scan", [&]<typename T>() {
+    hipLaunchKernelGGL(mingru_scan_kernel<T>, grid, dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(out.data_ptr()), reinterpret_cast<const T*>(z.data_ptr()),
+                       reinterpret_cast<const T*>(u.data_ptr()), reinterpret_cast<const T*>(g.data_ptr()),
+                       z.stride(0), z_b.data_ptr<float>(), u_b.data_ptr<float>(),
+                       state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(),
+                       fresh.data_ptr<int>(), n);
+  });
+}
+
+// x [T, C] row-strided; weight [C, K] fp32; tail [slots, K-1, C] fp32.
+void causal_conv_silu(at::Tensor out, at::Tensor x, at::Tensor weight, at::Tensor bias,
+                      at::Tensor tail, at::Tensor cu, at::Tensor slots, at::Tensor fresh) {
+  HY_GPU(x);
+  HY_INNER(x);
+  TORCH_CHECK(x.dim() == 2);
+  const long T_ = x.size(0);
+  const int C = x.size(1);
+  if (T_ == 0) return;
+  HY_F32(weight); HY_F32(bias);
+  TORCH_CHECK(weight.dim() == 2 && weight.size(0) == C && bias.numel() == C);
+  const int K = weight.size(1);
+  TORCH_CHECK(K >= 1 && K <= kConvMaxTaps, "1 to ", kConvMaxTaps, " taps");
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes() && out.scalar_type() == x.scalar_type());
+  const SeqDims d = seq_check(cu, slots, fresh, tail);
+  TORCH_CHECK(tail.dim() == 3 && tail.size(1) == K - 1 && tail.size(2) == C, "tail [slots, K-1, C] fp32");
+  // few rows (single tokens): a thread per row; prompts: 32 rows per thread
+  const int rpt = T_ <= 512 ? 1 : 32;
+  const dim3 grid((C + 255) / 256, (T_ + rpt - 1) / rpt);
+  hy_dispatch(x, "causal_conv_silu", [&]<typename T>() {
+    hipLaunchKernelGGL(causal_conv_silu_kernel<T>, grid, dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(out.data_ptr()), reinterpret_cast<const T*>(x.data_ptr()),
+                       x.stride(0), weight.data_ptr<float>(), bias.data_ptr<float>(),
+                       tail.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(),
+                       fresh.data_ptr<int>(), d.B, C, K, rpt);
+    if (K > 1)
+      hipLaunchKernelGGL(conv_tail_update_kernel<T>, dim3((C + 255) / 256, d.B), dim3(256), 0,
+                         hy_stream(), reinterpret_cast<const T*>(x.data_ptr()), x.stride(0),
+                         tail.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(),
+                         fresh.data_ptr<int>(), C, K);
+  });
+}
+
+// x [T, C] contiguous or row-strided, dt [T, C], z [T, C] row-strided, Bm / Cm
+// [T, N] row-strided slices of one projection output; state [slots, C, N].
+void selective_scan(at::Tensor out, at::Tensor x, at::Tensor dt, at::Tensor dt_b, at::Tensor A,
+                    at::Tensor Bm, at::Tensor Cm, at::Tensor D, at::Tensor z, at::Tensor state,
+                    at::Tensor cu, at::Tensor slots, at::Tensor fresh) {
+  HY_GPU(x);
+  HY_INNER(x); HY_INNER(dt); HY_INNER(z); HY_INNER(Bm); HY_INNER(Cm);
+  TORCH_CHECK(x.dim() == 2 && dt.sizes() == x.sizes() && z.sizes() == x.sizes());
+  const long T_ = x.size(0);
+  const int C = x.size(1);
+  if (T_ == 0) return;
+  TORCH_CHECK(Bm.dim() == 2 && Bm.size(0) == T_ && Cm.sizes() == Bm.sizes() &&
+              Bm.stride(0) == Cm.stride(0));
+  const int N = Bm.size(1);
+  HY_F32(dt_b); HY_F32(A); HY_F32(D);
+  TORCH_CHECK(dt_b.numel() == C && D.numel() == C && A.dim() == 2 && A.size(0) == C && A.size(1) == N);
+  const auto ty = x.scalar_type();
+  TORCH_CHECK(dt.scalar_type() == ty && z.scalar_type() == ty && Bm.scalar_type() == ty &&
+              Cm.scalar_type() == ty && out.scalar_type() == ty);
+  TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes());
+  const SeqDims d = seq_check(cu, slots, fresh, state);
+  TORCH_CHECK(state.dim() == 3 && state.size(1) == C && state.size(2) == N, "state [slots, C, N] fp32");
+  TORCH_CHECK(N >= 1 && N <= 1024, "1 to 1024 states per channel");
+  // NS states per lane, LPC lanes per channel (both powers of two)
+  int ns = 1;
+  while (ns < N && ns < 16) ns *= 2;
+  int lpc = 1;
+  while (ns * lpc < N) lpc *= 2;
+  const long threads = (long)C * lpc;
+  const dim3 grid((threads + 255) / 256, d.B);
+  const size_t lds = sizeof(float) * (size_t)kScanTT * 2 * N;
+  hy_dispatch(x, "selective_scan", [&]<typename T>() {
+    auto launch = [&]<int NS>() {
+      auto kern = selective_scan_kernel<T, NS>;
+      allow_lds(kern, lds);
+      hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(), reinterpret_cast<T*>(out.data_ptr()),
+                         reinterpret_cast<const T*>(x.data_ptr()), x.stride(0),
+                         reinterpret_cast<const T*>(dt.data_ptr()), dt.stride(0),
+                         dt_b.data_ptr<float>(), A.data_ptr<float>(),
+                         reinterpret_cast<const T*>(Bm.data_ptr()),
+                         reinterpret_cast<const T*>(Cm.data_ptr()), Bm.stride(0),
+                         D.data_ptr<float>(), reinterpret_cast<const T*>(z.data_ptr()), z.stride(0),
+                         state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(),
+                         fresh.data_ptr<int>(), C, N, lpc);
+    };
+    if (ns == 16) launch.template operator()<16>();
+    else if (ns == 8) launch.template operator()<8>();
+    else if (ns == 4) launch.template operator()<4>();
+    else if (ns == 2) launch.template operator()<2>();
+    else launch.template operator()<1>();
+  });
+}
+
+void softmax_topk(at::Tensor idx, at::Tensor w, at::Tensor logits, int64_t top, double scale) {
+  HY_GPU(logits);
+  TORCH_CHECK(logits.dim() == 2 && logits.is_contiguous() && logits.scalar_type() == at::kFloat,
+              "router logits must be fp32 [T, E]");
+  const long rows = logits.size(0);
+  const int E = logits.size(1);
+  if (rows == 0) return;
+  TORCH_CHECK(top >= 1 && top <= E && E <= 64 * 32, "top must be within 1..E, E at most 2048");
+  HY_I32(idx);
+  TORCH_CHECK(idx.dim() == 2 && idx.size(0) == rows && idx.size(1) == top);
+  TORCH_CHECK(w.scalar_type() == at::kFloat && w.is_contiguous() && w.sizes() == idx.sizes());
+  hipLaunchKernelGGL(softmax_topk_kernel, dim3((rows + 3) / 4), dim3(256), 0, hy_stream(),
+                     idx.data_ptr<int>(), w.data_ptr<float>(), logits.data_ptr<float>(), rows, E,
+                     (int)top, (float)scale);
+}
+
+void clamp_swish_mul(at::Tensor out, at::Tensor in, double limit) {
+  HY_GPU(in);
+  TORCH_CHECK(in.is_contiguous() && out.is_contiguous() && in.scalar_type() == out.scalar_type());
+  const int d = out.size(-1);
+  TORCH_CHECK(in.size(-1) == 2 * d, "in must be [..., 2*d]");
+  const long rows = out.numel() / d;
+  if (rows == 0) return;
+  if (in.scalar_type() == at::kBFloat16 && d % 8 == 0) {
+    using bf = __hip_bfloat16;
+    const long chunks = rows * (d / 8);
+    const int grid = (int)std::min<long>((chunks + 255) / 256, 4096);
+    hipLaunchKernelGGL(clamp_swish_mul_vec_kernel, dim3(grid), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<bf*>(out.data_ptr()), reinterpret_cast<const bf*>(in.data_ptr()),
+                       rows, d, (float)limit);
+    return;
+  }
+  hy_dispatch(in, "clamp_swish_mul", [&]<typename T>() {
+    const int grid = (int)std::min<long>((rows * d + 255) / 256, 4096);
+    hipLaunchKernelGGL(clamp_swish_mul_kernel<T>, dim3(grid), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(out.data_ptr()), reinterpret_cast<const T*>(in.data_ptr()),
+                       rows, d, (float)limit);
   });
 }
 
@@ -659,17 +986,26 @@ TORCH_LIBRARY(llmq_amd_hybrid, m) {
   m.def("sandwich_norm_res32(Tensor(a!) x, Tensor(b!) residual, Tensor w_post, Tensor w_pre, float eps, float offset) -> ()");
   m.def("act_and_mul(Tensor(a!) out, Tensor input, bool gelu) -> ()");
   m.def("qknorm_vmix_cache(Tensor(a!) q, Tensor k, Tensor v, Tensor q_w, Tensor k_w, Tensor? v_first, float lam, Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor slots, float eps) -> ()");
-  m.def("paged_attn_prefill(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor cu_q, Tensor q_start, int max_q, int span, float scale, int mask_mode, int pos_stride) -> ()");
-  m.def("paged_attn_decode(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor context_lens, int span, float scale, int mask_mode) -> ()");
+  m.def("paged_attn_prefill(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor cu_q, Tensor q_start, int max_q, int span, float scale, int mask_mode, int pos_stride, int bias_mode) -> ()");
+  m.def("paged_attn_decode(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor context_lens, int span, float scale, int mask_mode, int bias_mode) -> ()");
   m.def("gla_recurrence(Tensor(a!) o, Tensor q, Tensor? k, Tensor v, Tensor z, Tensor z_bias, Tensor(b!) state, Tensor cu, Tensor slots, Tensor fresh, float tau, Tensor? lower, bool q_silu, float q_scale) -> ()");
   m.def("gla_out_norm_gate(Tensor(a!) out, Tensor o, Tensor weight, Tensor? gate, float eps) -> ()");
   m.def("latent_rope_pack(Tensor(a!) out, Tensor q, Tensor q_lat, Tensor ckr, Tensor c_w, Tensor inv_freq, Tensor positions, Tensor(b!) k_cache, Tensor slots, int dim, int rot_dims, bool interleaved, float eps) -> ()");
   m.def("gated_residual_add(Tensor(a!) out, Tensor(b!) res, Tensor y1, Tensor g1, Tensor b1, Tensor? y2, Tensor? g2, Tensor? b2) -> ()");
   m.def("side_gate_mul(Tensor(a!) out, Tensor a, Tensor table, Tensor tokens, int offset) -> ()");
   m.def("sigmoid_topk(Tensor(a!) idx, Tensor(b!) w, Tensor logits, int top) -> ()");
-  m.def("moe_gate_up_gemv(Tensor(a!) hmid, Tensor h, Tensor idx, Tensor w, Tensor gate_up) -> ()");
-  m.def("moe_down_gemv(Tensor(a!) y, Tensor hmid, Tensor idx, Tensor down) -> ()");
-  m.def("moe_expert_gemv(Tensor(a!) out, Tensor input, Tensor idx, Tensor? w, Tensor weight, bool gate_up) -> ()");
+  m.def("moe_gate_up_gemv(Tensor(a!) hmid, Tensor h, Tensor idx, Tensor? w, Tensor gate_up, int act, float limit) -> ()");
+  m.def("moe_down_gemv(Tensor(a!) y, Tensor hmid, Tensor idx, Tensor down, Tensor? wo) -> ()");
+  m.def("moe_expert_gemv(Tensor(a!) out, Tensor input, Tensor idx, Tensor? w, Tensor weight, bool gate_up, int act, float limit) -> ()");
+  m.def("embed_sinusoid(Tensor(a!) out, Tensor embedding, Tensor ids, Tensor positions, Tensor inv_freq) -> ()");
+  m.def("scaled_add_norm(Tensor(a!) out, Tensor(b!) res, Tensor y, Tensor? y2, float a1, float a2, Tensor weight, float eps) -> ()");
+  m.def("depth_mix_norm(Tensor(a!) out, Tensor(b!) stack, int n, Tensor coef, Tensor y, Tensor? y2, float a1, float a2, Tensor weight, float eps) -> ()");
+  m.def("kv_scatter(Tensor k, Tensor v, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor slots) -> ()");
+  m.def("mingru_scan(Tensor(a!) out, Tensor z, Tensor u, Tensor g, Tensor z_b, Tensor u_b, Tensor(b!) state, Tensor cu, Tensor slots, Tensor fresh) -> ()");
+  m.def("causal_conv_silu(Tensor(a!) out, Tensor x, Tensor weight, Tensor bias, Tensor(b!) tail, Tensor cu, Tensor slots, Tensor fresh) -> ()");
+  m.def("selective_scan(Tensor(a!) out, Tensor x, Tensor dt, Tensor dt_b, Tensor A, Tensor Bm, Tensor Cm, Tensor D, Tensor z, Tensor(b!) state, Tensor cu, Tensor slots, Tensor fresh) -> ()");
+  m.def("softmax_topk(Tensor(a!) idx, Tensor(b!) w, Tensor logits, int top, float scale) -> ()");
+  m.def("clamp_swish_mul(Tensor(a!) out, Tensor input, float limit) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(llmq_amd_hybrid, CUDA, m) {
@@ -688,4 +1024,13 @@ TORCH_LIBRARY_IMPL(llmq_amd_hybrid, CUDA, m) {
   m.impl("moe_expert_gemv", &moe_expert_gemv);
   m.impl("gla_recurrence", &gla_recurrence);
   m.impl("gla_out_norm_gate", &gla_out_norm_gate);
+  m.impl("embed_sinusoid", &embed_sinusoid);
+  m.impl("scaled_add_norm", &scaled_add_norm);
+  m.impl("depth_mix_norm", &depth_mix_norm);
+  m.impl("kv_scatter", &kv_scatter);
+  m.impl("mingru_scan", &mingru_scan);
+  m.impl("causal_conv_silu", &causal_conv_silu);
+  m.impl("selective_scan", &selective_scan);
+  m.impl("softmax_topk", &softmax_topk);
+  m.impl("clamp_swish_mul", &clamp_swish_mul);
 }

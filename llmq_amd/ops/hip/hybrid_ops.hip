@@ -5,4 +5,5 @@
 #include "elementwise.hip"
 #include "seqmix.hip"
 #include "latent_moe.hip"
+#include "scan_mix.hip"
 #include "hybrid_bindings.cpp"

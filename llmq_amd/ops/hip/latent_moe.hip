@@ -248,18 +248,34 @@ DEVINL float wave_dot(const T* __restrict__ wrow, const float* __restrict__ x, i
 
 constexpr int kMoeRowsPerWave = 4;
 
-// hmid[r, f] = silu(gate_e[f] . x) * (up_e[f] . x);  gate_up [E, 2F, W]
+// What an expert does between its two projections. Plain: silu(g) * u.
+// Clamped: g = min(g, limit), u = clamp(u, +-limit), g * sigmoid(1.702 g) * (u + 1).
+constexpr int kMoeActSilu = 0;
+constexpr int kMoeActClampSwish = 1;
+
+DEVINL float moe_gated_act(float g, float u, int act, float limit) {
+  if (act == kMoeActClampSwish) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+  }
+  return g / (1.0f + expf(-g)) * u;
+}
+
+// hmid[r, f] = act(gate_e[f] . x, up_e[f] . x);  gate_up [E, 2F, W]; a null w
+// leaves the input unscaled (x = h[t])
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_gemv_kernel(
     T* __restrict__ hmid, const T* __restrict__ h, const int* __restrict__ idx,
-    const float* __restrict__ w, const T* __restrict__ gate_up, int top, int W, int F, int E) {
+    const float* __restrict__ w, const T* __restrict__ gate_up, int top, int W, int F, int E,
+    int act, float limit) {
   extern __shared__ float xs[];   // [W]
   const long r = blockIdx.y;
   const long t = r / top;
   const int e = min(max(idx[r], 0), E - 1);
-  const float wr = w[r];
+  const float wr = w ? w[r] : 1.0f;
   for (int i = threadIdx.x; i < W; i += blockDim.x)
-    xs[i] = to_f32(from_f32<T>(wr * to_f32(h[t * W + i])));
+    xs[i] = w ? to_f32(from_f32<T>(wr * to_f32(h[t * W + i]))) : to_f32(h[t * W + i]);
   __syncthreads();
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
   const T* ge = gate_up + (long)e * 2 * F * W;
@@ -267,15 +283,16 @@ __global__ __launch_bounds__(256) void moe_gate_up_gemv_kernel(
   for (int f = f0; f < min(F, f0 + kMoeRowsPerWave); ++f) {
     const float g = to_f32(from_f32<T>(wave_dot(ge + (long)f * W, xs, W, lane)));
     const float u = to_f32(from_f32<T>(wave_dot(ge + (long)(F + f) * W, xs, W, lane)));
-    if (lane == 0) hmid[r * F + f] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+    if (lane == 0) hmid[r * F + f] = from_f32<T>(moe_gated_act(g, u, act, limit));
   }
 }
 
-// y[t, c] = sum_k down_{e(t,k)}[c] . hmid[t*top + k];  down [E, W, F]
+// y[t, c] = sum_k wo[t, k] * (down_{e(t,k)}[c] . hmid[t*top + k]);  down [E, W, F];
+// a null wo weights every chosen expert's output with 1
 template <typename T>
 __global__ __launch_bounds__(256) void moe_down_gemv_kernel(
     T* __restrict__ y, const T* __restrict__ hmid, const int* __restrict__ idx,
-    const T* __restrict__ down, int top, int W, int F, int E) {
+    const T* __restrict__ down, int top, int W, int F, int E, const float* __restrict__ wo) {
   extern __shared__ float hs[];   // [top][F]
   const long t = blockIdx.y;
   for (int i = threadIdx.x; i < top * F; i += blockDim.x) hs[i] = to_f32(hmid[t * top * F + i]);
@@ -286,7 +303,8 @@ __global__ __launch_bounds__(256) void moe_down_gemv_kernel(
     float acc = 0.f;
     for (int k = 0; k < top; ++k) {
       const T* de = down + ((long)min(max(idx[t * top + k], 0), E - 1) * W + c) * F;
-      acc += to_f32(from_f32<T>(wave_dot(de, hs + k * F, F, lane)));
+      const float dk = to_f32(from_f32<T>(wave_dot(de, hs + k * F, F, lane)));
+      acc += wo ? wo[t * top + k] * dk : dk;
     }
     if (lane == 0) y[t * W + c] = from_f32<T>(acc);
   }
@@ -298,8 +316,8 @@ __global__ __launch_bounds__(256) void moe_down_gemv_kernel(
 // no host round trip, no sort) and runs them in chunks of kMoeTB rows, so a
 // weight row is read once per chunk instead of once per row. Inputs of a
 // chunk sit in LDS in the model dtype; accumulation is fp32.
-//   GATE_UP: weight [E, 2F, K], x[r] = round(w[r] * h[r / top]), out hmid[r, f] =
-//            silu(gate_f . x) * (up_f . x)
+//   GATE_UP: weight [E, 2F, K], x[r] = round(w[r] * h[r / top]) (h[r / top] when
+//            w is null), out hmid[r, f] = act(gate_f . x, up_f . x)
 //   else   : weight [E, N, K], x[r] = in[r], out[r, n] = weight_n . x
 constexpr int kMoeTB = 8;        // rows per chunk
 constexpr int kMoeFPW = 2;       // output features per wave and pass
@@ -308,7 +326,8 @@ constexpr int kMoeMaxRows = 2048;
 template <typename T, bool GATE_UP>
 __global__ __launch_bounds__(256) void moe_expert_gemv_kernel(
     T* __restrict__ out, const T* __restrict__ in, const int* __restrict__ idx,
-    const float* __restrict__ w, const T* __restrict__ weight, int rows, int top, int K, int N) {
+    const float* __restrict__ w, const T* __restrict__ weight, int rows, int top, int K, int N,
+    int act, float limit) {
   extern __shared__ __align__(16) unsigned char moe_smem[];
   __shared__ int count;
   int* list = reinterpret_cast<int*>(moe_smem);                 // [kMoeMaxRows]
@@ -333,8 +352,9 @@ __global__ __launch_bounds__(256) void moe_expert_gemv_kernel(
       float v = 0.f;
       if (tt < nt) {
         const int r = list[c0 + tt];
-        v = GATE_UP ? to_f32(from_f32<T>(w[r] * to_f32(in[(long)(r / top) * K + k])))
-                    : to_f32(in[(long)r * K + k]);
+        v = !GATE_UP ? to_f32(in[(long)r * K + k])
+            : w ? to_f32(from_f32<T>(w[r] * to_f32(in[(long)(r / top) * K + k])))
+                : to_f32(in[(long)(r / top) * K + k]);
       }
       xs[i] = from_f32<T>(v);
     }
@@ -390,7 +410,7 @@ __global__ __launch_bounds__(256) void moe_expert_gemv_kernel(
         g = to_f32(from_f32<T>(g));
         if (GATE_UP) {
           u = to_f32(from_f32<T>(u));
-          out[r * N + f] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+          out[r * N + f] = from_f32<T>(moe_gated_act(g, u, act, limit));
         } else {
           out[r * N + f] = from_f32<T>(g);
         }

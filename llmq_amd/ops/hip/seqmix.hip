@@ -237,6 +237,21 @@ DEVINL int mask_first_key(int pos, int span, int mode) {
   return mode == kMaskBlock ? (pos / span) * span : max(0, pos - span + 1);
 }
 
+// What a score gains for the distance d = i - j >= 0 of query and key.
+// Table: bias[h, min(d, bias_len - 1)], a learned value per distance. Log:
+// bias[h] = (r1, r2) and the score loses r1 * ln(1 + r2 * d).
+constexpr int kBiasTable = 0;
+constexpr int kBiasLog = 1;
+
+DEVINL float log_dist_bias(const float* __restrict__ r12, int d) {
+  return -r12[0] * log1pf(r12[1] * (float)d);
+}
+
+DEVINL float dist_bias(const float* __restrict__ bias, int bias_len, int mode, int h, int d) {
+  if (mode == kBiasLog) return log_dist_bias(bias + 2 * h, d);
+  return bias[(long)h * bias_len + min(d, bias_len - 1)];
+}
+
 template <typename T, int NV>
 __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     T* __restrict__ out, long out_stride,
@@ -248,7 +263,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     const int* __restrict__ cu_q,          // [B+1]
     const int* __restrict__ q_start,       // [B] position of a sequence's first query
     int H, int G, int D, int DV, int block_size, int span, float scale,
-    int v_row, int mask_mode) {
+    int v_row, int mask_mode, int bias_mode) {
   extern __shared__ float smem[];
   const int b = blockIdx.z, h = blockIdx.y;
   const int row0 = cu_q[b];
@@ -324,7 +339,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
       const bool vis = lane < nk && (w * 4 + r) < rows && key <= i &&
                        key >= mask_first_key(i, span, mask_mode);
       const float sc = !vis ? -INFINITY
-          : bias ? s[r] + bias[(long)h * bias_len + min(i - key, bias_len - 1)] : s[r];
+          : bias ? s[r] + dist_bias(bias, bias_len, bias_mode, h, i - key) : s[r];
       const float tmax = wave_reduce_max(sc);
       const float m_new = fmaxf(m[r], tmax);
       float p = 0.f, corr = 1.f;
@@ -405,7 +420,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
     int H, int G, int D, int DV, int block_size, int span, float scale,
-    int v_row, int mask_mode, int ps, int n_split, float* __restrict__ part) {
+    int v_row, int mask_mode, int ps, int n_split, float* __restrict__ part, int bias_mode) {
   // n_split > 1: the grid's y dimension carries (key split, head); a
   // workgroup walks only its share of the key tiles and writes its
   // unnormalised output, running maximum and sum to `part`
@@ -465,7 +480,8 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
   const int wave_lo = mask_first_key(wave_first, span, mask_mode);
   const bool wave_rows = w * 16 < rows;
   const int* bt = block_tables + (long)b * bt_stride;
-  const float* bias_h = bias ? bias + (long)h * bias_len : nullptr;
+  const bool bias_log = bias_mode == kBiasLog;
+  const float* bias_h = bias ? bias + (bias_log ? 2L * h : (long)h * bias_len) : nullptr;
   short* Pw = Ps + w * 2 * 16 * kMfmaKP;
   const bool v_vec = (DV % 8) == 0 && (v_row % 8) == 0;
 
@@ -532,7 +548,9 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     if (tid < 127) {
       // distances this tile can ask for: (pos0 + r) - (kt + c), r, c in [0, 64)
       const int d = pos0 - kt - 63 + tid;
-      Bs[tid] = (bias_h && d >= 0 && d < bias_len) ? bias_h[d] : 0.f;
+      Bs[tid] = !bias_h || d < 0 ? 0.f
+          : bias_log ? log_dist_bias(bias_h, d)
+          : d < bias_len ? bias_h[d] : 0.f;
     }
     __syncthreads();
     if (kt + kMfmaKT <= key_end) fetch(kt + kMfmaKT);
@@ -698,7 +716,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ context_lens,
     int H, int G, int D, int DV, int block_size, int span, float scale,
-    int v_row, int mask_mode) {
+    int v_row, int mask_mode, int bias_mode) {
   extern __shared__ __align__(16) float smem[];
   const int h0 = blockIdx.x * HPW, b = blockIdx.y;
   const int g = h0 / (H / G);
@@ -763,8 +781,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
       }
 #pragma unroll
       for (int hh = 0; hh < HPW; ++hh)
-        sc[hh] = bias ? s[hh] + bias[(long)(h0 + hh) * bias_len + min(i - key, bias_len - 1)]
-                      : s[hh];
+        sc[hh] = bias ? s[hh] + dist_bias(bias, bias_len, bias_mode, h0 + hh, i - key) : s[hh];
     }
     float p[HPW];
 #pragma unroll

@@ -384,10 +384,11 @@ def gla_out_norm_gate(o, weight, gate, eps, out_dtype):
 # forget-gate recurrences, gated parallel residuals and expert mixtures.
 
 
-def _window_attend(qb, kc, vc, pos, window, scale):
+def _window_attend(qb, kc, vc, pos, window, scale, log_bias=None):
     """qb [n, H, D] at absolute positions pos [n]; kc [L, G, D], vc [L, G, DV]
     cached keys/values of positions 0..L-1. Query i sees key j iff j <= i
-    and (window == 0 or i - j < window)."""
+    and (window == 0 or i - j < window). log_bias [H, 2] = (r1, r2) per head
+    takes r1 * ln(1 + r2 * (i - j)) off the scaled score."""
     n, H, _ = qb.shape
     G = kc.shape[1]
     lo = max(0, int(pos[0]) - window + 1) if window else 0
@@ -399,11 +400,16 @@ def _window_attend(qb, kc, vc, pos, window, scale):
     if window:
         vis = vis & (i - j < window)
     scores = torch.einsum("ihd,jhd->hij", qb.float(), kk) * scale
+    if log_bias is not None:
+        dist = (i - j).clamp(min=0).float().unsqueeze(0)
+        r1, r2 = log_bias[:, 0].float().view(-1, 1, 1), log_bias[:, 1].float().view(-1, 1, 1)
+        scores = scores - r1 * torch.log1p(r2 * dist)
     scores = scores.masked_fill(~vis.unsqueeze(0), float("-inf"))
     return torch.einsum("hij,jhd->ihd", torch.softmax(scores, dim=-1), vv)
 
 
-def window_attn_prefill(q, k_cache, v_cache, dv, block_tables, cu_q, q_start, window, scale):
+def window_attn_prefill(q, k_cache, v_cache, dv, block_tables, cu_q, q_start, window, scale,
+                        log_bias=None):
     """Causal / sliding-window softmax attention of packed prompt portions
     over the paged cache. v_cache None: a key row's first dv channels are
     its value."""
@@ -418,11 +424,12 @@ def window_attn_prefill(q, k_cache, v_cache, dv, block_tables, cu_q, q_start, wi
         kc = _gather_seq(k_cache, block_tables[b], L)
         vc = kc[..., :dv] if v_cache is None else _gather_seq(v_cache, block_tables[b], L)
         pos = torch.arange(p0, L, device=q.device)
-        out[s:e] = _window_attend(q[s:e], kc, vc, pos, window, scale).to(q.dtype)
+        out[s:e] = _window_attend(q[s:e], kc, vc, pos, window, scale, log_bias).to(q.dtype)
     return out
 
 
-def window_attn_decode(q, k_cache, v_cache, dv, block_tables, context_lens, window, scale):
+def window_attn_decode(q, k_cache, v_cache, dv, block_tables, context_lens, window, scale,
+                       log_bias=None):
     B, H, _ = q.shape
     out = q.new_empty(B, H, dv)
     for b in range(B):
@@ -430,7 +437,8 @@ def window_attn_decode(q, k_cache, v_cache, dv, block_tables, context_lens, wind
         kc = _gather_seq(k_cache, block_tables[b], L)
         vc = kc[..., :dv] if v_cache is None else _gather_seq(v_cache, block_tables[b], L)
         pos = torch.tensor([L - 1], device=q.device)
-        out[b : b + 1] = _window_attend(q[b : b + 1], kc, vc, pos, window, scale).to(q.dtype)
+        out[b : b + 1] = _window_attend(q[b : b + 1], kc, vc, pos, window, scale,
+                                        log_bias).to(q.dtype)
     return out
 
 
@@ -531,3 +539,145 @@ def sigmoid_topk(logits, top):
     s = torch.sigmoid(logits.float())
     w, idx = torch.topk(s, top, dim=-1)
     return idx.to(torch.int32), w
+
+
+# ------------------------------ scan hybrids (minGRU / selective scan) ref --
+# Reference forms of the ops added for decoders built from elementwise gated
+# recurrences, selective scans beside attention, softmax-routed clamped
+# experts and a learned average over layer outputs.
+
+
+def sinusoid_inv_freq(width: int) -> torch.Tensor:
+    """fp32 table 10000^(-2i/width), one entry per (sin, cos) pair, rounded
+    once from float64."""
+    i = torch.arange((width + 1) // 2, dtype=torch.float64)
+    return torch.pow(torch.tensor(10000.0, dtype=torch.float64), -2.0 * i / width).float()
+
+
+def embed_sinusoid(embedding, ids, positions, inv_freq):
+    """fp32 [T, W]: embedding[ids] plus the sinusoidal position vector, entry
+    2i = sin(p * inv_freq[i]), entry 2i+1 = cos of the same angle (fp32)."""
+    x = embedding[ids].float()
+    W = x.shape[1]
+    ang = positions.float().unsqueeze(1) * inv_freq.float().unsqueeze(0)
+    pe = torch.stack([torch.sin(ang), torch.cos(ang)], dim=-1).reshape(x.shape[0], -1)[:, :W]
+    return x + pe
+
+
+def scaled_add_norm(res, y, y2, a1, a2, weight, eps, out_dtype):
+    """res (fp32, in place) += a1 * y [+ a2 * y2]; returns rmsnorm(res) * weight."""
+    add = a1 * y.float()
+    if y2 is not None:
+        add = add + a2 * y2.float()
+    res.add_(add)
+    return rmsnorm_cast(res, weight, eps, 0.0, out_dtype)
+
+
+def depth_mix_norm(stack, n, coef, y, y2, a1, a2, weight, eps, out_dtype):
+    """stack [>= n+1, T, W] fp32 holds the embedding output and the layer
+    results so far in rows 0..n-1. Row n-1 (in place) += a1 * y [+ a2 * y2];
+    row n = sum_j coef[j] * row j (j < n); returns rmsnorm(row n) * weight."""
+    add = a1 * y.float()
+    if y2 is not None:
+        add = add + a2 * y2.float()
+    stack[n - 1].add_(add)
+    mix = torch.einsum("j,jtw->tw", coef.float()[:n], stack[:n])
+    stack[n].copy_(mix)
+    return rmsnorm_cast(stack[n], weight, eps, 0.0, out_dtype)
+
+
+def kv_scatter(k, v, k_cache, v_cache, slots):
+    """k [T, G*D], v [T, G*DV] scattered into the paged cache rows `slots`
+    (negative: skipped)."""
+    G, bs, D = k_cache.shape[1], k_cache.shape[2], k_cache.shape[3]
+    DV = v_cache.shape[3]
+    keep = slots >= 0
+    s = slots[keep].long()
+    k_cache[s // bs, :, s % bs, :] = k[keep].reshape(-1, G, D).to(k_cache.dtype)
+    v_cache[s // bs, :, s % bs, :] = v[keep].reshape(-1, G, DV).to(v_cache.dtype)
+
+
+def mingru_scan(z, u, g, z_b, u_b, state, cu, slots, fresh, out_dtype):
+    """minGRU over packed sequences. z, u, g [T, n] projections; gate
+    a = sigmoid(z + z_b), candidate c = u' + 1/2 (u' >= 0) or sigmoid(u')
+    with u' = u + u_b; S <- (1 - a) S + a c per channel (fp32 state
+    [slots, n], advanced in place, zero start where fresh); returns
+    S_t * silu(g_t) in out_dtype."""
+    a = torch.sigmoid(z.float() + z_b.float())
+    uu = u.float() + u_b.float()
+    c = torch.where(uu >= 0, uu + 0.5, torch.sigmoid(uu))
+    out = torch.empty(z.shape, dtype=torch.float32, device=z.device)
+    for b in range(len(slots)):
+        s, e = int(cu[b]), int(cu[b + 1])
+        slot = int(slots[b])
+        S = torch.zeros_like(state[slot]) if int(fresh[b]) else state[slot].clone()
+        for t in range(s, e):
+            S = (1.0 - a[t]) * S + a[t] * c[t]
+            out[t] = S
+        state[slot] = S
+    return (out * torch.nn.functional.silu(g.float())).to(out_dtype)
+
+
+def causal_conv_silu(x, weight, bias, tail, cu, slots, fresh):
+    """Per-channel causal convolution + SiLU over packed sequences.
+    x [T, C]; weight [C, K] fp32 (last column = the current token's tap);
+    bias [C] fp32; tail [slots, K-1, C] fp32 holds each sequence's last K-1
+    inputs (zeros before the start), advanced in place. Returns [T, C] in
+    x's dtype."""
+    K = weight.shape[1]
+    out = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    xf = x.float()
+    for b in range(len(slots)):
+        s, e = int(cu[b]), int(cu[b + 1])
+        slot = int(slots[b])
+        past = torch.zeros_like(tail[slot]) if int(fresh[b]) else tail[slot].clone()
+        seq = torch.cat([past, xf[s:e]], dim=0)          # [K-1 + n, C]
+        n = e - s
+        acc = bias.float().unsqueeze(0).expand(n, -1).clone()
+        for k in range(K):
+            acc += seq[k:k + n] * weight[:, k].float()
+        out[s:e] = acc
+        if K > 1:
+            tail[slot] = seq[seq.shape[0] - (K - 1):]
+    return torch.nn.functional.silu(out).to(x.dtype)
+
+
+def selective_scan(x, dt, dt_b, A, Bm, Cm, D, z, state, cu, slots, fresh):
+    """Selective scan over packed sequences. x, dt, z [T, C]; Bm, Cm [T, N];
+    dt_b, D [C] fp32; A [C, N] fp32 (negative); state [slots, C, N] fp32
+    advanced in place. step = softplus(dt + dt_b);
+    S <- exp(step A) S + step x B;  y = S C + D x;  returns y * silu(z)."""
+    step = torch.nn.functional.softplus(dt.float() + dt_b.float())
+    xf, Bf, Cf = x.float(), Bm.float(), Cm.float()
+    y = torch.empty(x.shape, dtype=torch.float32, device=x.device)
+    for b in range(len(slots)):
+        s, e = int(cu[b]), int(cu[b + 1])
+        slot = int(slots[b])
+        S = torch.zeros_like(state[slot]) if int(fresh[b]) else state[slot].clone()
+        for t in range(s, e):
+            S = torch.exp(step[t].unsqueeze(1) * A) * S \
+                + (step[t] * xf[t]).unsqueeze(1) * Bf[t].unsqueeze(0)
+            y[t] = S @ Cf[t] + D * xf[t]
+        state[slot] = S
+    return (y * torch.nn.functional.silu(z.float())).to(x.dtype)
+
+
+def softmax_topk(logits, top, scale):
+    """Router: scores = softmax(logits) over all experts (fp32); the `top`
+    largest per row, times scale. Returns (indices int32, weights fp32)."""
+    s = torch.softmax(logits.float(), dim=-1)
+    w, idx = torch.topk(s, top, dim=-1)
+    return idx.to(torch.int32), w * scale
+
+
+def clamp_swish_mul(x, limit):
+    """[*, 2d] -> g * sigmoid(1.702 g) * (u + 1) with g = min(x[..., :d], limit)
+    and u = clamp(x[..., d:], -limit, limit)."""
+    d = x.shape[-1] // 2
+    g = x[..., :d].float().clamp(max=limit)
+    u = x[..., d:].float().clamp(-limit, limit)
+    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)).to(x.dtype)
+
+
+def softcap(x, cap):
+    return cap * torch.tanh(x.float() / cap)
