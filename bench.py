@@ -44,7 +44,8 @@ def compare_hybrid(args) -> None:
     models = args.compare_models.split(",")
     batch, prompt_len = min(args.batch, 64), args.prompt_len
     if not use_gpu:
-        tiny = ["tiny-kosalorn"] if args.compare_kosalorn else []
+        tiny = ["tiny-muvetar", "tiny-kosalorn"] if args.compare_muvetar else \
+            ["tiny-kosalorn"] if args.compare_kosalorn else []
         models, batch, prompt_len = tiny + ["tiny-kakovik", "tiny-llama"], 4, 48
     for name in models:
         engine = LLMEngine(EngineConfig(
@@ -137,12 +138,19 @@ def main() -> None:
                         help="the same comparison for the Kosalorn looped-hybrid presets "
                         "(latent attention, HGRN2, expert mixtures) beside the Kakovik "
                         "and Llama presets of equal layer sizes")
+    parser.add_argument("--compare-muvetar", action="store_true",
+                        help="the same comparison for the Muvetar scan/attention presets "
+                        "(minGRU, selective scan beside attention, softmax-routed experts) "
+                        "beside the Kosalorn expert-mixture preset and the Llama presets of "
+                        "equal layer sizes")
     args = parser.parse_args()
+    if args.compare_models is None and args.compare_muvetar:
+        args.compare_models = "muvetar-1b,kosalorn-1b-moe,llama-3.2-1b,muvetar-3b,kosalorn-3b,llama-3.2-3b"
     if args.compare_models is None:
         args.compare_models = (
             "kosalorn-1b,kosalorn-1b-moe,kakovik-1b,llama-3.2-1b,kosalorn-3b,kakovik-3b,llama-3.2-3b"
             if args.compare_kosalorn else "kakovik-1b,llama-3.2-1b,kakovik-3b,llama-3.2-3b")
-    if args.compare_hybrid or args.compare_kosalorn:
+    if args.compare_hybrid or args.compare_kosalorn or args.compare_muvetar:
         compare_hybrid(args)
         return
 

@@ -842,14 +842,31 @@ void mingru_scan(at::Tensor out, at::Tensor z, at::Tensor u, at::Tensor g, at::T
   TORCH_CHECK(z_b.numel() == n && u_b.numel() == n);
   const SeqDims d = seq_check(cu, slots, fresh, state);
   TORCH_CHECK(state.dim() == 2 && state.size(1) == n, "state [slots, n] fp32");
-  const dim3 grid((n + 255) / 256, d.B);
+  // long portions run parallel over time: 16 (or 4) chunks per sequence
+  const long avg = T_ / std::max(1, d.B);
   hy_dispatch(z, "mingru_scan", [&]<typename T>() {
-    hipLaunchKernelGGL(mingru_scan_kernel<T>, grid, dim3(256), 0, hy_stream(),
-                       reinterpret_cast<T*>(out.data_ptr()), reinterpret_cast<const T*>(z.data_ptr()),
-                       reinterpret_cast<const T*>(u.data_ptr()), reinterpret_cast<const T*>(g.data_ptr()),
-                       z.stride(0), z_b.data_ptr<float>(), u_b.data_ptr<float>(),
-                       state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(),
-                       fresh.data_ptr<int>(), n);
+    auto launch = [&]<int NC>() {
+      if constexpr (NC == 1) {
+        hipLaunchKernelGGL(mingru_scan_kernel<T>, dim3((n + 255) / 256, d.B), dim3(256), 0,
+                           hy_stream(), reinterpret_cast<T*>(out.data_ptr()),
+                           reinterpret_cast<const T*>(z.data_ptr()),
+                           reinterpret_cast<const T*>(u.data_ptr()),
+                           reinterpret_cast<const T*>(g.data_ptr()), z.stride(0),
+                           z_b.data_ptr<float>(), u_b.data_ptr<float>(), state.data_ptr<float>(),
+                           cu.data_ptr<int>(), slots.data_ptr<int>(), fresh.data_ptr<int>(), n);
+      } else {
+        hipLaunchKernelGGL((mingru_scan_chunked_kernel<T, NC>), dim3((n + 63) / 64, d.B),
+                           dim3(64 * NC), 0, hy_stream(), reinterpret_cast<T*>(out.data_ptr()),
+                           reinterpret_cast<const T*>(z.data_ptr()),
+                           reinterpret_cast<const T*>(u.data_ptr()),
+                           reinterpret_cast<const T*>(g.data_ptr()), z.stride(0),
+                           z_b.data_ptr<float>(), u_b.data_ptr<float>(), state.data_ptr<float>(),
+                           cu.data_ptr<int>(), slots.data_ptr<int>(), fresh.data_ptr<int>(), n);
+      }
+    };
+    if (avg >= 128) launch.template operator()<16>();
+    else if (avg >= 16) launch.template operator()<4>();
+    else launch.template operator()<1>();
   });
 }
 
@@ -914,14 +931,18 @@ void selective_scan(at::Tensor out, at::Tensor x, at::Tensor dt, at::Tensor dt_b
   while (ns < N && ns < 16) ns *= 2;
   int lpc = 1;
   while (ns * lpc < N) lpc *= 2;
-  const long threads = (long)C * lpc;
-  const dim3 grid((threads + 255) / 256, d.B);
-  const size_t lds = sizeof(float) * (size_t)kScanTT * 2 * N;
+  // long portions run parallel over time: 8 chunks per sequence
+  const bool chunked = T_ / std::max(1, d.B) >= 64;
+  const int nc = chunked ? 8 : 1;
+  const dim3 grid(((long)C * lpc + 63) / 64, d.B);
+  const size_t lds = sizeof(float) * ((size_t)nc * kScanTT * 2 * N +
+                                      (chunked ? (size_t)nc * 64 * (1 + ns) : 0));
   hy_dispatch(x, "selective_scan", [&]<typename T>() {
-    auto launch = [&]<int NS>() {
-      auto kern = selective_scan_kernel<T, NS>;
+    auto launch = [&]<int NS, int NC>() {
+      auto kern = selective_scan_kernel<T, NS, NC>;
       allow_lds(kern, lds);
-      hipLaunchKernelGGL(kern, grid, dim3(256), lds, hy_stream(), reinterpret_cast<T*>(out.data_ptr()),
+      hipLaunchKernelGGL(kern, grid, dim3(64 * NC), lds, hy_stream(),
+                         reinterpret_cast<T*>(out.data_ptr()),
                          reinterpret_cast<const T*>(x.data_ptr()), x.stride(0),
                          reinterpret_cast<const T*>(dt.data_ptr()), dt.stride(0),
                          dt_b.data_ptr<float>(), A.data_ptr<float>(),
@@ -931,11 +952,15 @@ void selective_scan(at::Tensor out, at::Tensor x, at::Tensor dt, at::Tensor dt_b
                          state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(),
                          fresh.data_ptr<int>(), C, N, lpc);
     };
-    if (ns == 16) launch.template operator()<16>();
-    else if (ns == 8) launch.template operator()<8>();
-    else if (ns == 4) launch.template operator()<4>();
-    else if (ns == 2) launch.template operator()<2>();
-    else launch.template operator()<1>();
+    auto by_ns = [&]<int NC>() {
+      if (ns == 16) launch.template operator()<16, NC>();
+      else if (ns == 8) launch.template operator()<8, NC>();
+      else if (ns == 4) launch.template operator()<4, NC>();
+      else if (ns == 2) launch.template operator()<2, NC>();
+      else launch.template operator()<1, NC>();
+    };
+    if (chunked) by_ns.template operator()<8>();
+    else by_ns.template operator()<1>();
   });
 }
 

@@ -275,6 +275,81 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(
   *st = S;
 }
 
+// The same recurrence for long portions, parallel over time: a workgroup owns
+// 64 channels of one sequence and NC contiguous chunks of its tokens, one
+// wave per chunk. A linear recurrence S <- (1 - a) S + a c composes: a chunk
+// is summarised by (P, E) = (product of its 1 - a, its end state from a zero
+// start). Pass 1 computes every chunk's (P, E); a chunk's start state then
+// follows from the sequence's start state and the summaries before it; pass 2
+// walks the chunk again from that start and writes the outputs.
+template <typename T, int NC>
+__global__ __launch_bounds__(64 * NC) void mingru_scan_chunked_kernel(
+    T* __restrict__ out, const T* __restrict__ z, const T* __restrict__ u,
+    const T* __restrict__ g, long in_stride, const float* __restrict__ z_b,
+    const float* __restrict__ u_b, float* __restrict__ state, const int* __restrict__ cu,
+    const int* __restrict__ slots, const int* __restrict__ fresh, int n) {
+  __shared__ float Ps[NC][64], Es[NC][64];
+  constexpr bool FAST = sizeof(T) == 2;
+  const int b = blockIdx.y;
+  const int lane = threadIdx.x & 63, k = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
+  const int s = cu[b], e = cu[b + 1];
+  if (e <= s) return;
+  const bool live = c < n;
+  const int cc = live ? c : 0;
+  const int L = (e - s + NC - 1) / NC;
+  const int t_lo = min(e, s + k * L), t_hi = min(e, t_lo + L);
+  const float zb = z_b[cc], ub = u_b[cc];
+  auto sig = [](float v) { return 1.0f / (1.0f + (FAST ? __expf(-v) : expf(-v))); };
+  float P = 1.f, E = 0.f;
+  for (int t0 = t_lo; t0 < t_hi; t0 += kGruPre) {
+    float zv[kGruPre], uv[kGruPre];
+#pragma unroll
+    for (int i = 0; i < kGruPre; ++i) {
+      const long r = (long)min(t0 + i, t_hi - 1) * in_stride + cc;
+      zv[i] = to_f32(z[r]);
+      uv[i] = to_f32(u[r]);
+    }
+#pragma unroll
+    for (int i = 0; i < kGruPre; ++i) {
+      if (t0 + i < t_hi) {
+        const float a = sig(zv[i] + zb);
+        const float uu = uv[i] + ub;
+        const float cand = uu >= 0.f ? uu + 0.5f : sig(uu);
+        E = (1.0f - a) * E + a * cand;
+        P *= 1.0f - a;
+      }
+    }
+  }
+  Ps[k][lane] = P;
+  Es[k][lane] = E;
+  __syncthreads();
+  float* st = state + (long)slots[b] * n + cc;
+  float S = fresh[b] ? 0.f : *st;
+  for (int kk = 0; kk < k; ++kk) S = Ps[kk][lane] * S + Es[kk][lane];
+  for (int t0 = t_lo; t0 < t_hi; t0 += kGruPre) {
+    float zv[kGruPre], uv[kGruPre], gv[kGruPre];
+#pragma unroll
+    for (int i = 0; i < kGruPre; ++i) {
+      const long r = (long)min(t0 + i, t_hi - 1) * in_stride + cc;
+      zv[i] = to_f32(z[r]);
+      uv[i] = to_f32(u[r]);
+      gv[i] = to_f32(g[r]);
+    }
+#pragma unroll
+    for (int i = 0; i < kGruPre; ++i) {
+      if (t0 + i < t_hi) {
+        const float a = sig(zv[i] + zb);
+        const float uu = uv[i] + ub;
+        const float cand = uu >= 0.f ? uu + 0.5f : sig(uu);
+        S = (1.0f - a) * S + a * cand;
+        if (live) out[(long)(t0 + i) * n + c] = from_f32<T>(S * gv[i] * sig(gv[i]));
+      }
+    }
+  }
+  if (live && k == NC - 1) *st = S;   // the last chunk ends where the portion ends
+}
+
 // ------------------------------------------------ short causal convolution --
 // out[t, c] = silu(b[c] + sum_k w[c, k] * V[j - (K-1) + k]) for row t = s + j
 // of a sequence whose inputs are V[j >= 0] = x[s + j] and V[-(K-1) .. -1] =
@@ -283,6 +358,7 @@ __global__ __launch_bounds__(256) void mingru_scan_kernel(
 // consecutive packed rows, wherever they fall in their sequences. The tail is
 // advanced by a second kernel after every read of the old one has happened.
 constexpr int kConvMaxTaps = 8;
+constexpr int kConvGroup = 8;    // rows whose inputs a thread fetches together
 
 template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
@@ -303,41 +379,52 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
   int b = 0;
   while (cu[b + 1] <= r0) ++b;   // the sequence of row r0 (empty sequences skipped)
   bool load_window = true;
-  for (int r = r0; r < r1; ++r) {
-    while (cu[b + 1] <= r) {
-      ++b;
-      load_window = true;
-    }
-    if (load_window) {
-      const int s = cu[b], j = r - s;
-      const float* tl = tail + (long)slots[b] * (K - 1) * C + c;
-      const bool fr = fresh[b] != 0;
-      // win[k] = V[j - (K-1) + k], k < K-1
+  for (int g0 = r0; g0 < r1; g0 += kConvGroup) {
+    // the group's own inputs first: independent loads, all in flight at once
+    float xg[kConvGroup];
 #pragma unroll
-      for (int k = 0; k < kConvMaxTaps - 1; ++k) {
-        if (k < K - 1) {
-          const int jj = j - (K - 1) + k;
-          win[k] = jj >= 0 ? to_f32(x[(long)(s + jj) * x_stride + c])
-                           : (fr ? 0.f : tl[(long)(jj + K - 1) * C]);
+    for (int i = 0; i < kConvGroup; ++i)
+      xg[i] = to_f32(x[(long)min(g0 + i, r1 - 1) * x_stride + c]);
+#pragma unroll
+    for (int i = 0; i < kConvGroup; ++i) {
+      const int r = g0 + i;
+      if (r < r1) {
+        while (cu[b + 1] <= r) {
+          ++b;
+          load_window = true;
         }
+        if (load_window) {
+          const int s = cu[b], j = r - s;
+          const float* tl = tail + (long)slots[b] * (K - 1) * C + c;
+          const bool fr = fresh[b] != 0;
+          // win[k] = V[j - (K-1) + k], k < K-1
+#pragma unroll
+          for (int k = 0; k < kConvMaxTaps - 1; ++k) {
+            if (k < K - 1) {
+              const int jj = j - (K - 1) + k;
+              win[k] = jj >= 0 ? to_f32(x[(long)(s + jj) * x_stride + c])
+                               : (fr ? 0.f : tl[(long)(jj + K - 1) * C]);
+            }
+          }
+          load_window = false;
+        }
+        const float xv = xg[i];
+        float acc = bc;
+#pragma unroll
+        for (int k = 0; k < kConvMaxTaps - 1; ++k)
+          if (k < K - 1) acc += wk[k] * win[k];
+#pragma unroll
+        for (int k = 0; k < kConvMaxTaps; ++k)
+          if (k == K - 1) acc += wk[k] * xv;
+        out[(long)r * C + c] = from_f32<T>(acc * sigmoid_f(acc));
+#pragma unroll
+        for (int k = 0; k < kConvMaxTaps - 2; ++k)
+          if (k < K - 2) win[k] = win[k + 1];
+#pragma unroll
+        for (int k = 0; k < kConvMaxTaps - 1; ++k)
+          if (k == K - 2) win[k] = xv;
       }
-      load_window = false;
     }
-    const float xv = to_f32(x[(long)r * x_stride + c]);
-    float acc = bc;
-#pragma unroll
-    for (int k = 0; k < kConvMaxTaps - 1; ++k)
-      if (k < K - 1) acc += wk[k] * win[k];
-#pragma unroll
-    for (int k = 0; k < kConvMaxTaps; ++k)
-      if (k == K - 1) acc += wk[k] * xv;
-    out[(long)r * C + c] = from_f32<T>(acc * sigmoid_f(acc));
-#pragma unroll
-    for (int k = 0; k < kConvMaxTaps - 2; ++k)
-      if (k < K - 2) win[k] = win[k + 1];
-#pragma unroll
-    for (int k = 0; k < kConvMaxTaps - 1; ++k)
-      if (k == K - 2) win[k] = xv;
   }
 }
 
@@ -375,82 +462,134 @@ __global__ __launch_bounds__(256) void conv_tail_update_kernel(
 //   S[c, n] <- exp(step * A[c, n]) * S[c, n] + step * x[t, c] * B[t, n]
 //   y[t, c] = sum_n S[c, n] * C[t, n] + D[c] * x[t, c];  out = y * silu(z[t, c])
 // state [slots, C, N] fp32, advanced in place; a fresh sequence starts from
-// zero without reading its slot. A workgroup owns 256 / LPC channels of one
-// sequence: LPC lanes share a channel, each with NS of its states in
-// registers (state index sub * NS + j). B and C of kScanTT tokens are staged
-// in LDS as fp32 and read as broadcasts; a channel's x, dt and z of those
-// tokens are fetched before the serial part.
+// zero without reading its slot.
+//
+// A workgroup owns 64 / LPC channels of one sequence and NC contiguous chunks
+// of its tokens, one wave per chunk: LPC adjacent lanes share a channel, each
+// with NS of its states in registers (state index sub * NS + j). The
+// recurrence is linear in S, so a chunk is summarised by the sum of its steps
+// (its decay is exp(A * that sum)) and its end state from a zero start. Pass 1
+// computes the summaries, a chunk's start state follows from the sequence's
+// start state and the summaries before it, pass 2 walks the chunk again from
+// there and writes the outputs. NC = 1 (single tokens, short portions) is the
+// plain serial walk. B and C of kScanTT tokens per wave are staged in LDS as
+// fp32 and read as broadcasts; a channel's x, dt and z of those tokens are
+// fetched before the serial part. bf16 models use the hardware exp/log; fp32
+// models the accurate functions.
 constexpr int kScanTT = 8;
 
-DEVINL float softplus_f(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+template <bool FAST>
+DEVINL float scan_exp(float x) { return FAST ? __expf(x) : expf(x); }
 
-template <typename T, int NS>
-__global__ __launch_bounds__(256) void selective_scan_kernel(
+template <bool FAST>
+DEVINL float scan_softplus(float x) {
+  if (x > 20.f) return x;
+  return FAST ? __logf(1.0f + __expf(x)) : log1pf(expf(x));
+}
+
+template <typename T, int NS, int NC>
+__global__ __launch_bounds__(64 * NC) void selective_scan_kernel(
     T* __restrict__ out, const T* __restrict__ x, long x_stride, const T* __restrict__ dt,
     long dt_stride, const float* __restrict__ dt_b, const float* __restrict__ A,
     const T* __restrict__ Bm, const T* __restrict__ Cm, long bc_stride,
     const float* __restrict__ Dp, const T* __restrict__ z, long z_stride,
     float* __restrict__ state, const int* __restrict__ cu, const int* __restrict__ slots,
     const int* __restrict__ fresh, int C, int N, int lpc) {
-  extern __shared__ float scan_smem[];   // [kScanTT][2][N]
+  // [NC][kScanTT][2][N] staged B and C rows, then (NC > 1) the chunk
+  // summaries: [NC][64] step sums and [NC][NS][64] end states
+  extern __shared__ float scan_smem[];
+  constexpr bool FAST = sizeof(T) == 2;
   const int b = blockIdx.y;
   const int s = cu[b], e = cu[b + 1];
   if (e <= s) return;
-  const int tid = threadIdx.x;
-  const int c = (blockIdx.x * 256 + tid) / lpc, sub = tid % lpc;
+  const int lane = threadIdx.x & 63, k = threadIdx.x >> 6;
+  const int c = (blockIdx.x * 64 + lane) / lpc, sub = lane % lpc;
   const bool live = c < C;
+  const int cc = live ? c : 0;
   const int n0 = sub * NS;
+  float* bc = scan_smem + (long)k * kScanTT * 2 * N;
+  float* sums = scan_smem + (long)NC * kScanTT * 2 * N;   // [NC][64]
+  float* ends = sums + NC * 64;                            // [NC][NS][64]
+  const int L = (e - s + NC - 1) / NC;                     // tokens per chunk
+  const int t_lo = min(e, s + k * L), t_hi = min(e, t_lo + L);
   float S[NS], a[NS];
-  float* st = state + ((long)slots[b] * C + (live ? c : 0)) * N;
+  float* st = state + ((long)slots[b] * C + cc) * N;
   const bool fr = fresh[b] != 0;
 #pragma unroll
-  for (int j = 0; j < NS; ++j) {
-    const bool ok = live && n0 + j < N;
-    a[j] = ok ? A[(long)c * N + n0 + j] : 0.f;
-    S[j] = (ok && !fr) ? st[n0 + j] : 0.f;
-  }
-  const float db = live ? dt_b[c] : 0.f, dd = live ? Dp[c] : 0.f;
-  for (int t0 = s; t0 < e; t0 += kScanTT) {
-    const int nt = min(kScanTT, e - t0);
-    __syncthreads();
-    for (int i = tid; i < nt * N; i += 256) {
-      const int tt = i / N, n = i % N;
-      scan_smem[(tt * 2) * N + n] = to_f32(Bm[(long)(t0 + tt) * bc_stride + n]);
-      scan_smem[(tt * 2 + 1) * N + n] = to_f32(Cm[(long)(t0 + tt) * bc_stride + n]);
-    }
-    float xv[kScanTT], dv[kScanTT], zv[kScanTT];
+  for (int j = 0; j < NS; ++j) a[j] = (live && n0 + j < N) ? A[(long)cc * N + n0 + j] : 0.f;
+  const float db = dt_b[cc], dd = Dp[cc];
+
+  // one pass over the chunk; OUT = false computes only the state
+  auto walk = [&]<bool OUT>(float& step_sum) {
+    for (int t0 = t_lo; t0 < t_lo + L; t0 += kScanTT) {   // same trip count in every wave
+      const int nt = max(0, min(kScanTT, t_hi - t0));
+      __syncthreads();
+      for (int i = lane; i < nt * N; i += 64) {
+        const int tt = i / N, n = i % N;
+        bc[(tt * 2) * N + n] = to_f32(Bm[(long)(t0 + tt) * bc_stride + n]);
+        if (OUT) bc[(tt * 2 + 1) * N + n] = to_f32(Cm[(long)(t0 + tt) * bc_stride + n]);
+      }
+      float xv[kScanTT], sp[kScanTT], zg[kScanTT];
 #pragma unroll
-    for (int tt = 0; tt < kScanTT; ++tt) {
-      const long r = min(t0 + tt, e - 1);
-      xv[tt] = live ? to_f32(x[r * x_stride + c]) : 0.f;
-      dv[tt] = live ? to_f32(dt[r * dt_stride + c]) : 0.f;
-      zv[tt] = live ? to_f32(z[r * z_stride + c]) : 0.f;
-    }
-    __syncthreads();
-#pragma unroll
-    for (int tt = 0; tt < kScanTT; ++tt) {
-      if (tt < nt) {
-        const float step = softplus_f(dv[tt] + db);
-        const float xs = step * xv[tt];
-        const float* bs = scan_smem + (tt * 2) * N + n0;
-        const float* cs = bs + N;
-        float acc = 0.f;
-#pragma unroll
-        for (int j = 0; j < NS; ++j) {
-          if (n0 + j < N) {
-            S[j] = expf(step * a[j]) * S[j] + xs * bs[j];
-            acc += S[j] * cs[j];
-          }
+      for (int tt = 0; tt < kScanTT; ++tt) {
+        const long r = max(min(t0 + tt, t_hi - 1), s);
+        xv[tt] = to_f32(x[r * x_stride + cc]);
+        sp[tt] = scan_softplus<FAST>(to_f32(dt[r * dt_stride + cc]) + db);
+        if (OUT) {
+          const float zz = to_f32(z[r * z_stride + cc]);
+          zg[tt] = zz / (1.0f + scan_exp<FAST>(-zz));
         }
-        for (int off = 1; off < lpc; off <<= 1) acc += __shfl_xor(acc, off, WAVE);
-        if (live && sub == 0) {
-          const float yv = acc + dd * xv[tt];
-          out[(long)(t0 + tt) * C + c] = from_f32<T>(yv * zv[tt] * sigmoid_f(zv[tt]));
+      }
+      __syncthreads();
+#pragma unroll
+      for (int tt = 0; tt < kScanTT; ++tt) {
+        if (tt < nt) {
+          const float step = sp[tt];
+          const float xs = step * xv[tt];
+          const float* bs = bc + (tt * 2) * N + n0;
+          const float* cs = bs + N;
+          step_sum += step;
+          float acc = 0.f;
+#pragma unroll
+          for (int j = 0; j < NS; ++j) {
+            if (n0 + j < N) {
+              S[j] = scan_exp<FAST>(step * a[j]) * S[j] + xs * bs[j];
+              if (OUT) acc += S[j] * cs[j];
+            }
+          }
+          if (OUT) {
+            for (int off = 1; off < lpc; off <<= 1) acc += __shfl_xor(acc, off, WAVE);
+            if (live && sub == 0)
+              out[(long)(t0 + tt) * C + c] = from_f32<T>((acc + dd * xv[tt]) * zg[tt]);
+          }
         }
       }
     }
+  };
+
+  if constexpr (NC > 1) {
+#pragma unroll
+    for (int j = 0; j < NS; ++j) S[j] = 0.f;
+    float step_sum = 0.f;
+    walk.template operator()<false>(step_sum);
+    sums[k * 64 + lane] = step_sum;
+#pragma unroll
+    for (int j = 0; j < NS; ++j) ends[(k * NS + j) * 64 + lane] = S[j];
+    __syncthreads();
   }
-  if (live) {
+#pragma unroll
+  for (int j = 0; j < NS; ++j) S[j] = (live && !fr && n0 + j < N) ? st[n0 + j] : 0.f;
+  if constexpr (NC > 1) {
+    for (int kk = 0; kk < k; ++kk) {
+      const float ssum = sums[kk * 64 + lane];
+#pragma unroll
+      for (int j = 0; j < NS; ++j)
+        S[j] = scan_exp<FAST>(ssum * a[j]) * S[j] + ends[(kk * NS + j) * 64 + lane];
+    }
+  }
+  float unused = 0.f;
+  walk.template operator()<true>(unused);
+  if (live && k == NC - 1) {   // the last chunk ends where the portion ends
 #pragma unroll
     for (int j = 0; j < NS; ++j)
       if (n0 + j < N) st[n0 + j] = S[j];

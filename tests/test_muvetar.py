@@ -550,6 +550,40 @@ def test_mingru_op_keeps_a_far_input(target, n):
 
 
 @pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("lens", [[200, 1, 3, 130], [1, 1, 1], [17, 40], [700]])
+def test_mingru_op_unequal_sequences_in_one_call(target, lens):
+    """Long and very short sequences side by side (the long ones run split
+    over time), strided inputs, a state carried in from an earlier call."""
+    device, dtype = dev_dtype(target)
+    C, T = 70, sum(lens)
+    g = torch.Generator().manual_seed(T)
+    p = (torch.randn(T, 3 * C + 5, generator=g) * 1.5).to(dtype)
+    zb, ub = torch.randn(C, generator=g), torch.randn(C, generator=g) * 0.5
+    start = torch.randn(len(lens) + 1, C, generator=g)
+    fresh = [i % 2 for i in range(len(lens))]
+    slots = list(range(len(lens), 0, -1))
+    cu, sl, fr = _seq_meta(lens, slots, fresh, device)
+    state = start.clone().to(device)
+    pd = p.to(device)
+    got = ops.mingru_scan(pd[:, 1:C + 1], pd[:, C + 2:2 * C + 2], pd[:, 2 * C + 3:3 * C + 3],
+                          zb.to(device), ub.to(device), state, cu, sl, fr, dtype).double().cpu()
+    pz, pu, pg = (p[:, a:a + C].double() for a in (1, C + 2, 2 * C + 3))
+    at = 0
+    tol = 3e-2 if dtype == torch.bfloat16 else 1e-4
+    for b, n in enumerate(lens):
+        S = torch.zeros(C, dtype=torch.float64) if fresh[b] else start[slots[b]].double()
+        for t in range(at, at + n):
+            a = oracle.sigmoid(pz[t] + zb.double())
+            uu = pu[t] + ub.double()
+            S = (1 - a) * S + a * torch.where(uu >= 0, uu + 0.5, oracle.sigmoid(uu))
+            want = S * oracle.silu(pg[t])
+            assert (got[t] - want).abs().max() < tol * max(1.0, float(want.abs().max())), (b, t)
+        assert (state[slots[b]].double().cpu() - S).abs().max() < 1e-4
+        at += n
+    assert torch.equal(state[0].cpu(), start[0])
+
+
+@pytest.mark.parametrize("target", DEVICES)
 @pytest.mark.parametrize("C,K", [(5, 4), (64, 3), (300, 8), (7, 2), (9, 1)])
 def test_conv_op_across_cuts_shorter_than_its_reach(target, C, K):
     device, dtype = dev_dtype(target)
@@ -603,7 +637,7 @@ def _scan_reference(x, dt, dt_b, A, Bm, Cm, D, z):
 def test_selective_scan_op_against_token_by_token(target, C, N):
     device, dtype = dev_dtype(target)
     g = torch.Generator().manual_seed(C + N)
-    T = 75
+    T = 380
     rn = lambda *s: torch.randn(*s, generator=g)
     x, dt, z = rn(T, C).to(dtype), (rn(T, C) - 1.0).to(dtype), rn(T, C).to(dtype)
     bc = rn(T, 2 * N + 3).to(dtype)
@@ -614,7 +648,7 @@ def test_selective_scan_op_against_token_by_token(target, C, N):
     state = torch.full((4, C, N), 9.0, device=device)
     dev = lambda t: t.to(device)
     outs, at = [], 0
-    for cut in (1, 2, 30, 1, 1, 40):
+    for cut in (1, 2, 30, 1, 1, 40, 205, 100):      # the long ones run split over time
         cu, slots, fresh = _seq_meta([cut], [3], [int(at == 0)], device)
         sl = slice(at, at + cut)
         outs.append(ops.selective_scan(dev(x[sl]), dev(dt[sl]), dev(dt_b), dev(A), dev(bc)[sl, 1:N + 1],
@@ -627,20 +661,21 @@ def test_selective_scan_op_against_token_by_token(target, C, N):
     assert (got - want).abs().max() < tol * scale
     assert (state[3].double().cpu() - S_end).abs().max() < tol * S_end.abs().max().clamp(min=1.0)
     assert float(state[0].min()) == 9.0 and float(state[2].max()) == 9.0
-    # three sequences in one call equal each alone
-    lens = [20, 1, 54]
-    cu, slots, fresh = _seq_meta(lens, [2, 0, 1], [1, 1, 1], device)
-    st = torch.zeros(4, C, N, device=device)
-    got = ops.selective_scan(dev(x), dev(dt), dev(dt_b), dev(A), dev(bc)[:, 1:N + 1],
-                             dev(bc)[:, N + 1:2 * N + 1], dev(D), dev(z), st, cu, slots,
-                             fresh).double().cpu()
-    at = 0
-    for n in lens:
-        sl = slice(at, at + n)
-        ref, _ = _scan_reference(x[sl].double(), dt[sl].double(), dt_b.double(), A.double(),
-                                 Bm[sl].double(), Cm[sl].double(), D.double(), z[sl].double())
-        assert (got[sl] - ref).abs().max() < tol * scale
-        at += n
+    # three sequences in one call equal each alone, short and long ones mixed
+    for lens in ([20, 1, 54], [300, 2, 78], [5, 370, 5]):
+        cu, slots, fresh = _seq_meta(lens, [2, 0, 1], [1, 1, 1], device)
+        st = torch.zeros(4, C, N, device=device)
+        n_all = sum(lens)
+        got = ops.selective_scan(dev(x)[:n_all], dev(dt)[:n_all], dev(dt_b), dev(A),
+                                 dev(bc)[:n_all, 1:N + 1], dev(bc)[:n_all, N + 1:2 * N + 1], dev(D),
+                                 dev(z)[:n_all], st, cu, slots, fresh).double().cpu()
+        at = 0
+        for n in lens:
+            sl = slice(at, at + n)
+            ref, _ = _scan_reference(x[sl].double(), dt[sl].double(), dt_b.double(), A.double(),
+                                     Bm[sl].double(), Cm[sl].double(), D.double(), z[sl].double())
+            assert (got[sl] - ref).abs().max() < tol * scale, lens
+            at += n
 
 
 @pytest.mark.parametrize("target", DEVICES)
