@@ -633,6 +633,10 @@ MOE_GEMV_MAX_ROWS = 64
 # row list's size) rows are grouped by expert inside the kernel
 MOE_GROUP_MIN_ROWS = 16
 MOE_GROUP_MAX_ROWS = 2048
+# from MOE_GROUP_MIN_ROWS rows on, while experts x tokens stays below this: the
+# dense form, every expert on every token as one batched GEMM pair (all
+# experts' weights are streamed anyway once the rows outnumber the experts)
+MOE_DENSE_MAX_PAIRS = 16384
 
 
 def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False, act: str = "silu",
@@ -644,15 +648,32 @@ def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False, act: str = "s
     with g = min(g, limit), u = clamp(u, +-limit).
     h [T, W]; idx/w [T, top]; gate_up [E, 2F, W]; down [E, W, F].
 
-    Few rows (or sync_free, for captured decode graphs): one matrix-vector
-    kernel pair that reads each row's expert weights. Many rows: rows
-    sorted by expert and one GEMM pair per expert on contiguous slices (the
-    per-expert row counts cross to the host once)."""
+    Few rows: one matrix-vector kernel pair that reads only each row's
+    expert weights. Decode batches (sync_free, for captured graphs) with
+    more rows than that: every expert runs on every token as one batched
+    GEMM pair on the matrix cores, and a token's unchosen experts weigh
+    nothing in the join. Many rows (prompt portions): rows sorted by expert
+    and one GEMM pair per expert on contiguous slices (the per-expert row
+    counts cross to the host once)."""
     T, top = idx.shape
     act_mode = _MOE_ACTS[act]
     if h.is_cuda and (sync_free or T * top <= MOE_GEMV_MAX_ROWS):
         _use_hybrid(h)
         F_ = down.shape[2]
+        E = gate_up.shape[0]
+        if T * top >= MOE_GROUP_MIN_ROWS and E * T <= MOE_DENSE_MAX_PAIRS:
+            wd = torch.zeros(T, E, dtype=torch.float32, device=h.device)
+            wd.scatter_(1, idx.long(), w)
+            if weight_output:
+                xs = h.unsqueeze(0).expand(E, T, h.shape[1])
+            else:  # zero input for the experts a token did not choose
+                xs = (h.float().unsqueeze(0) * wd.t().unsqueeze(-1)).to(h.dtype)
+            gu = torch.bmm(xs, gate_up.transpose(1, 2)).view(E * T, 2 * F_)
+            mid = act_and_mul(gu) if act == "silu" else clamp_swish_mul(gu, limit)
+            yk = torch.bmm(mid.view(E, T, F_), down.transpose(1, 2))
+            y = torch.empty_like(h)
+            _HY.moe_combine(y, yk, wd if weight_output else None)
+            return y
         hmid = torch.empty(T * top, F_, dtype=h.dtype, device=h.device)
         w_in = None if weight_output else w
         if MOE_GROUP_MIN_ROWS <= T * top <= MOE_GROUP_MAX_ROWS and \

@@ -331,12 +331,12 @@ void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Ten
   TORCH_CHECK(context_lens.numel() == B && block_tables.size(0) == B);
   // query heads per workgroup: as many of one kv head's as divide evenly
   const int per_kv = a.H / a.G;
-  int hpw = per_kv % 8 == 0 ? 8 : per_kv % 4 == 0 ? 4 : per_kv % 2 == 0 ? 2 : 1;
+  int hpw = per_kv % 8 == 0 ? 8 : per_kv % 4 == 0 ? 4 : per_kv % 3 == 0 ? 3 : per_kv % 2 == 0 ? 2 : 1;
   auto lds_for = [&](int n) {
     return sizeof(float) * ((size_t)n * ((a.D + 3) & ~3) + 2 * kDecWaves * n +
                             (size_t)kDecWaves * n * a.DV);
   };
-  while (hpw > 1 && lds_for(hpw) > 150 * 1024) hpw /= 2;   // wide heads: fewer per workgroup
+  while (hpw > 1 && lds_for(hpw) > 150 * 1024) hpw = hpw == 3 ? 1 : hpw / 2;   // wide heads: fewer per workgroup
   const size_t lds = lds_for(hpw);
   hy_dispatch(q, "paged_attn_decode", [&]<typename T>() {
     dispatch_nv(a.DV, [&]<int NV>() {
@@ -356,6 +356,7 @@ void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Ten
       };
       if (hpw == 8) launch.template operator()<8>();
       else if (hpw == 4) launch.template operator()<4>();
+      else if (hpw == 3) launch.template operator()<3>();
       else if (hpw == 2) launch.template operator()<2>();
       else launch.template operator()<1>();
     });
@@ -677,6 +678,28 @@ void moe_expert_gemv(at::Tensor out, at::Tensor in, at::Tensor idx, const std::o
   });
 }
 
+
+// yk [E, T, W] -> y [T, W] = sum_e wd[t, e] * yk[e, t] (wd null: plain sum)
+void moe_combine(at::Tensor y, at::Tensor yk, const std::optional<at::Tensor>& wd) {
+  HY_GPU(yk);
+  TORCH_CHECK(yk.dim() == 3 && yk.is_contiguous() && y.dim() == 2 && y.is_contiguous());
+  const int E = yk.size(0), W = yk.size(2);
+  const long rows = yk.size(1);
+  if (rows == 0) return;
+  TORCH_CHECK(y.size(0) == rows && y.size(1) == W && y.scalar_type() == yk.scalar_type());
+  const float* wp = nullptr;
+  if (wd.has_value()) {
+    TORCH_CHECK(wd->scalar_type() == at::kFloat && wd->is_contiguous() && wd->is_cuda() &&
+                wd->dim() == 2 && wd->size(0) == rows && wd->size(1) == E, "wd must be fp32 [T, E]");
+    wp = wd->data_ptr<float>();
+  }
+  const int grid = (int)std::min<long>((rows * W + 255) / 256, 4096);
+  hy_dispatch(yk, "moe_combine", [&]<typename T>() {
+    hipLaunchKernelGGL(moe_combine_kernel<T>, dim3(grid), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(y.data_ptr()), reinterpret_cast<const T*>(yk.data_ptr()),
+                       wp, rows, W, E);
+  });
+}
 
 // ---- scan/attention hybrids ------------------------------------------------
 
@@ -1022,6 +1045,7 @@ TORCH_LIBRARY(llmq_amd_hybrid, m) {
   m.def("moe_gate_up_gemv(Tensor(a!) hmid, Tensor h, Tensor idx, Tensor? w, Tensor gate_up, int act, float limit) -> ()");
   m.def("moe_down_gemv(Tensor(a!) y, Tensor hmid, Tensor idx, Tensor down, Tensor? wo) -> ()");
   m.def("moe_expert_gemv(Tensor(a!) out, Tensor input, Tensor idx, Tensor? w, Tensor weight, bool gate_up, int act, float limit) -> ()");
+  m.def("moe_combine(Tensor(a!) y, Tensor yk, Tensor? wd) -> ()");
   m.def("embed_sinusoid(Tensor(a!) out, Tensor embedding, Tensor ids, Tensor positions, Tensor inv_freq) -> ()");
   m.def("scaled_add_norm(Tensor(a!) out, Tensor(b!) res, Tensor y, Tensor? y2, float a1, float a2, Tensor weight, float eps) -> ()");
   m.def("depth_mix_norm(Tensor(a!) out, Tensor(b!) stack, int n, Tensor coef, Tensor y, Tensor? y2, float a1, float a2, Tensor weight, float eps) -> ()");
@@ -1049,6 +1073,7 @@ TORCH_LIBRARY_IMPL(llmq_amd_hybrid, CUDA, m) {
   m.impl("moe_expert_gemv", &moe_expert_gemv);
   m.impl("gla_recurrence", &gla_recurrence);
   m.impl("gla_out_norm_gate", &gla_out_norm_gate);
+  m.impl("moe_combine", &moe_combine);
   m.impl("embed_sinusoid", &embed_sinusoid);
   m.impl("scaled_add_norm", &scaled_add_norm);
   m.impl("depth_mix_norm", &depth_mix_norm);

@@ -418,3 +418,24 @@ __global__ __launch_bounds__(256) void moe_expert_gemv_kernel(
     }
   }
 }
+
+// --------------------------------- expert mixture, every expert on every row --
+// The join of the dense form (a batched GEMM pair that runs all E experts on
+// all rows): y[t, :] = sum_e wd[t, e] * yk[e, t, :], fp32 accumulation. wd is
+// the router's weights scattered into a dense [T, E] table, zero for experts
+// a token did not choose; a null wd sums the experts' outputs as they are.
+template <typename T>
+__global__ void moe_combine_kernel(T* __restrict__ y, const T* __restrict__ yk,
+                                   const float* __restrict__ wd, long rows, int W, int E) {
+  const long total = rows * W;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long t = idx / W;
+    float acc = 0.f;
+    for (int e = 0; e < E; ++e) {
+      const float v = to_f32(yk[(long)e * total + idx]);
+      acc += wd ? wd[t * E + e] * v : v;
+    }
+    y[idx] = from_f32<T>(acc);
+  }
+}

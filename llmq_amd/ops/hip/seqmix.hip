@@ -243,12 +243,16 @@ DEVINL int mask_first_key(int pos, int span, int mode) {
 constexpr int kBiasTable = 0;
 constexpr int kBiasLog = 1;
 
+// FAST (bf16 models): the hardware logarithm; fp32 models: log1pf.
+template <bool FAST>
 DEVINL float log_dist_bias(const float* __restrict__ r12, int d) {
-  return -r12[0] * log1pf(r12[1] * (float)d);
+  const float a = r12[1] * (float)d;
+  return -r12[0] * (FAST ? __logf(1.0f + a) : log1pf(a));
 }
 
+template <bool FAST>
 DEVINL float dist_bias(const float* __restrict__ bias, int bias_len, int mode, int h, int d) {
-  if (mode == kBiasLog) return log_dist_bias(bias + 2 * h, d);
+  if (mode == kBiasLog) return log_dist_bias<FAST>(bias + 2 * h, d);
   return bias[(long)h * bias_len + min(d, bias_len - 1)];
 }
 
@@ -339,7 +343,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
       const bool vis = lane < nk && (w * 4 + r) < rows && key <= i &&
                        key >= mask_first_key(i, span, mask_mode);
       const float sc = !vis ? -INFINITY
-          : bias ? s[r] + dist_bias(bias, bias_len, bias_mode, h, i - key) : s[r];
+          : bias ? s[r] + dist_bias<sizeof(T) == 2>(bias, bias_len, bias_mode, h, i - key) : s[r];
       const float tmax = wave_reduce_max(sc);
       const float m_new = fmaxf(m[r], tmax);
       float p = 0.f, corr = 1.f;
@@ -549,7 +553,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
       // distances this tile can ask for: (pos0 + r) - (kt + c), r, c in [0, 64)
       const int d = pos0 - kt - 63 + tid;
       Bs[tid] = !bias_h || d < 0 ? 0.f
-          : bias_log ? log_dist_bias(bias_h, d)
+          : bias_log ? log_dist_bias<true>(bias_h, d)
           : d < bias_len ? bias_h[d] : 0.f;
     }
     __syncthreads();
@@ -781,7 +785,8 @@ __global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
       }
 #pragma unroll
       for (int hh = 0; hh < HPW; ++hh)
-        sc[hh] = bias ? s[hh] + dist_bias(bias, bias_len, bias_mode, h0 + hh, i - key) : s[hh];
+        sc[hh] = bias ? s[hh] + dist_bias<sizeof(T) == 2>(bias, bias_len, bias_mode, h0 + hh, i - key)
+                      : s[hh];
     }
     float p[HPW];
 #pragma unroll
