@@ -357,7 +357,7 @@ __global__ __launch_bounds__(64 * NC) void mingru_scan_chunked_kernel(
 // sequence). Not a recurrence: a thread owns one channel and kConvRows
 // consecutive packed rows, wherever they fall in their sequences. The tail is
 // advanced by a second kernel after every read of the old one has happened.
-constexpr int kConvMaxTaps = 8;
+constexpr int kConvMaxTaps = 16;
 constexpr int kConvGroup = 8;    // rows whose inputs a thread fetches together
 
 template <typename T>
@@ -515,8 +515,20 @@ __global__ __launch_bounds__(64 * NC) void selective_scan_kernel(
   float S[NS], a[NS];
   float* st = state + ((long)slots[b] * C + cc) * N;
   const bool fr = fresh[b] != 0;
+  if (NS % 4 == 0 && N % 4 == 0) {
 #pragma unroll
-  for (int j = 0; j < NS; ++j) a[j] = (live && n0 + j < N) ? A[(long)cc * N + n0 + j] : 0.f;
+    for (int j = 0; j < NS / 4 * 4; j += 4) {
+      float4 av = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (live && n0 + j < N) av = *reinterpret_cast<const float4*>(A + (long)cc * N + n0 + j);
+      a[j] = av.x;
+      if (j + 1 < NS) a[j + 1] = av.y;
+      if (j + 2 < NS) a[j + 2] = av.z;
+      if (j + 3 < NS) a[j + 3] = av.w;
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < NS; ++j) a[j] = (live && n0 + j < N) ? A[(long)cc * N + n0 + j] : 0.f;
+  }
   const float db = dt_b[cc], dd = Dp[cc];
 
   // one pass over the chunk; OUT = false computes only the state
@@ -577,8 +589,22 @@ __global__ __launch_bounds__(64 * NC) void selective_scan_kernel(
     for (int j = 0; j < NS; ++j) ends[(k * NS + j) * 64 + lane] = S[j];
     __syncthreads();
   }
+  bool vec4 = false;   // a lane's states as 16-byte accesses
+  if constexpr (NS % 4 == 0) {
+    vec4 = N % 4 == 0;
+    if (vec4) {
 #pragma unroll
-  for (int j = 0; j < NS; ++j) S[j] = (live && !fr && n0 + j < N) ? st[n0 + j] : 0.f;
+      for (int j = 0; j < NS; j += 4) {
+        float4 sv = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live && !fr && n0 + j < N) sv = *reinterpret_cast<const float4*>(st + n0 + j);
+        S[j] = sv.x; S[j + 1] = sv.y; S[j + 2] = sv.z; S[j + 3] = sv.w;
+      }
+    }
+  }
+  if (!vec4) {
+#pragma unroll
+    for (int j = 0; j < NS; ++j) S[j] = (live && !fr && n0 + j < N) ? st[n0 + j] : 0.f;
+  }
   if constexpr (NC > 1) {
     for (int kk = 0; kk < k; ++kk) {
       const float ssum = sums[kk * 64 + lane];
@@ -590,9 +616,20 @@ __global__ __launch_bounds__(64 * NC) void selective_scan_kernel(
   float unused = 0.f;
   walk.template operator()<true>(unused);
   if (live && k == NC - 1) {   // the last chunk ends where the portion ends
+    if constexpr (NS % 4 == 0) {
+      if (vec4) {
 #pragma unroll
-    for (int j = 0; j < NS; ++j)
-      if (n0 + j < N) st[n0 + j] = S[j];
+        for (int j = 0; j < NS; j += 4)
+          if (n0 + j < N)
+            *reinterpret_cast<float4*>(st + n0 + j) =
+                make_float4(S[j], S[j + 1], S[j + 2], S[j + 3]);
+      }
+    }
+    if (!vec4) {
+#pragma unroll
+      for (int j = 0; j < NS; ++j)
+        if (n0 + j < N) st[n0 + j] = S[j];
+    }
   }
 }
 
