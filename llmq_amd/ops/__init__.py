@@ -709,6 +709,11 @@ def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False, act: str = "s
             at += n
     inv = torch.empty_like(order)
     inv[order] = torch.arange(order.numel(), device=order.device)
+    if h.is_cuda:
+        _use_hybrid(h)
+        y = torch.empty_like(h)
+        _HY.moe_gather_combine(y, ys, inv, w.contiguous() if weight_output else None, top)
+        return y
     yk = ys[inv].view(T, top, -1).float()
     if weight_output:
         yk = yk * w.unsqueeze(-1)

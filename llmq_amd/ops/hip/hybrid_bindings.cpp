@@ -701,6 +701,32 @@ void moe_combine(at::Tensor y, at::Tensor yk, const std::optional<at::Tensor>& w
   });
 }
 
+// ys [T*top, W] (expert-sorted rows), pos [T*top] int64 -> y [T, W]
+void moe_gather_combine(at::Tensor y, at::Tensor ys, at::Tensor pos,
+                        const std::optional<at::Tensor>& w, int64_t top) {
+  HY_GPU(ys);
+  TORCH_CHECK(ys.dim() == 2 && ys.is_contiguous() && y.dim() == 2 && y.is_contiguous());
+  const long rows = y.size(0);
+  const int W = y.size(1);
+  if (rows == 0) return;
+  TORCH_CHECK(top >= 1 && ys.size(0) == rows * top && ys.size(1) == W &&
+              y.scalar_type() == ys.scalar_type());
+  TORCH_CHECK(pos.scalar_type() == at::kLong && pos.is_contiguous() && pos.is_cuda() &&
+              pos.numel() == rows * top, "pos must be int64 [T * top]");
+  const float* wp = nullptr;
+  if (w.has_value()) {
+    TORCH_CHECK(w->scalar_type() == at::kFloat && w->is_contiguous() && w->is_cuda() &&
+                w->numel() == rows * top, "w must be fp32 [T, top]");
+    wp = w->data_ptr<float>();
+  }
+  const int grid = (int)std::min<long>((rows * W / 4 + 255) / 256 + 1, 8192);
+  hy_dispatch(ys, "moe_gather_combine", [&]<typename T>() {
+    hipLaunchKernelGGL(moe_gather_combine_kernel<T>, dim3(grid), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(y.data_ptr()), reinterpret_cast<const T*>(ys.data_ptr()),
+                       pos.data_ptr<long>(), wp, rows, (int)top, W);
+  });
+}
+
 // ---- scan/attention hybrids ------------------------------------------------
 
 #define HY_F32(x) TORCH_CHECK(x.scalar_type() == at::kFloat && x.is_contiguous() && x.is_cuda(), #x " must be contiguous fp32 on the GPU")
@@ -1046,6 +1072,7 @@ TORCH_LIBRARY(llmq_amd_hybrid, m) {
   m.def("moe_down_gemv(Tensor(a!) y, Tensor hmid, Tensor idx, Tensor down, Tensor? wo) -> ()");
   m.def("moe_expert_gemv(Tensor(a!) out, Tensor input, Tensor idx, Tensor? w, Tensor weight, bool gate_up, int act, float limit) -> ()");
   m.def("moe_combine(Tensor(a!) y, Tensor yk, Tensor? wd) -> ()");
+  m.def("moe_gather_combine(Tensor(a!) y, Tensor ys, Tensor pos, Tensor? w, int top) -> ()");
   m.def("embed_sinusoid(Tensor(a!) out, Tensor embedding, Tensor ids, Tensor positions, Tensor inv_freq) -> ()");
   m.def("scaled_add_norm(Tensor(a!) out, Tensor(b!) res, Tensor y, Tensor? y2, float a1, float a2, Tensor weight, float eps) -> ()");
   m.def("depth_mix_norm(Tensor(a!) out, Tensor(b!) stack, int n, Tensor coef, Tensor y, Tensor? y2, float a1, float a2, Tensor weight, float eps) -> ()");
@@ -1074,6 +1101,7 @@ TORCH_LIBRARY_IMPL(llmq_amd_hybrid, CUDA, m) {
   m.impl("gla_recurrence", &gla_recurrence);
   m.impl("gla_out_norm_gate", &gla_out_norm_gate);
   m.impl("moe_combine", &moe_combine);
+  m.impl("moe_gather_combine", &moe_gather_combine);
   m.impl("embed_sinusoid", &embed_sinusoid);
   m.impl("scaled_add_norm", &scaled_add_norm);
   m.impl("depth_mix_norm", &depth_mix_norm);

@@ -439,3 +439,49 @@ __global__ void moe_combine_kernel(T* __restrict__ y, const T* __restrict__ yk,
     y[idx] = from_f32<T>(acc);
   }
 }
+
+// The join of the sorted form (rows grouped by expert, one GEMM pair per
+// expert): y[t, :] = sum_k w[t, k] * ys[pos[t * top + k], :], where pos maps a
+// (token, choice) pair to its row in the expert-sorted order; fp32
+// accumulation; a null w sums the rows as they are.
+template <typename T>
+__global__ void moe_gather_combine_kernel(T* __restrict__ y, const T* __restrict__ ys,
+                                          const long* __restrict__ pos,
+                                          const float* __restrict__ w, long rows, int top, int W) {
+  constexpr int VE = Vec8<T>::kElems;
+  if (W % VE == 0) {
+    const int per_row = W / VE;
+    const long total = rows * per_row;
+    for (long gi = blockIdx.x * (long)blockDim.x + threadIdx.x; gi < total;
+         gi += (long)gridDim.x * blockDim.x) {
+      const long t = gi / per_row;
+      const int col = (int)(gi % per_row) * VE;
+      float acc[VE];
+#pragma unroll
+      for (int j = 0; j < VE; ++j) acc[j] = 0.f;
+      for (int k = 0; k < top; ++k) {
+        const Vec8<T> v = load16(ys + pos[t * top + k] * W + col);
+        const float wk = w ? w[t * top + k] : 1.0f;
+#pragma unroll
+        for (int j = 0; j < VE; ++j) acc[j] += wk * to_f32(v.data[j]);
+      }
+      Vec8<T> o;
+#pragma unroll
+      for (int j = 0; j < VE; ++j) o.data[j] = from_f32<T>(acc[j]);
+      store16(y + t * W + col, o);
+    }
+    return;
+  }
+  const long total = rows * W;
+  for (long idx = blockIdx.x * (long)blockDim.x + threadIdx.x; idx < total;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long t = idx / W;
+    const int col = (int)(idx % W);
+    float acc = 0.f;
+    for (int k = 0; k < top; ++k) {
+      const float v = to_f32(ys[pos[t * top + k] * W + col]);
+      acc += w ? w[t * top + k] * v : v;
+    }
+    y[idx] = from_f32<T>(acc);
+  }
+}
