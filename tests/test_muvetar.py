@@ -851,12 +851,14 @@ def test_decode_graph_replays_equal_eager(mixed_model):
     the replays, against the same steps run eagerly."""
     target = ("cuda", "float32")
     cfg, tensors, path = mixed_model(target)
+    # eight sequences: enough (token, expert) rows that the captured steps run
+    # the expert mixture in its dense batched form
     toks = {r: tokens_for(n, cfg["vocab"], 50 + i) for i, (r, n) in enumerate(
-        {"a": 30, "b": 12, "c": 19}.items())}
+        {"a": 30, "b": 12, "c": 19, "d": 9, "e": 25, "f": 14, "g": 11, "h": 21}.items())}
     results = []
     for eager in (True, False):
         device, dtype = target
-        eng = LLMEngine(EngineConfig(model=path, device=device, dtype=dtype, max_num_seqs=4,
+        eng = LLMEngine(EngineConfig(model=path, device=device, dtype=dtype, max_num_seqs=8,
                                      max_model_len=256, num_kv_blocks=32, enforce_eager=eager))
         assert eng.runner.use_graphs == (not eager)
         rows = []
