@@ -742,7 +742,7 @@ def muvetar_spec_from_config(cfg: dict, name: str) -> MuvetarSpec:
     for i, lc in enumerate(cfg["layers"]):
         mc, kind = lc["mixer"], lc["type"]
         if kind == "mingru":
-            mixer = MinGRUSpec(width=int(mc["width"]))
+            mixer = MinGRUSpec(width=int(mc.get("width", cfg["width"])))
         elif kind == "parallel":
             lt, rt = mc["left"], mc["right"]
             heads = int(lt["heads"])
