@@ -416,11 +416,10 @@ def test_long_decode_across_pages(mixed_model, target):
 
 def _needle_case(device, dtype, key_pos, query_pos, decode, r1, r2, H=2, G=1, D=16, DV=8,
                  block_size=16):
-    """All keys score 0 but the needle at key_pos, whose raw score is `boost`
-    chosen so that after the distance penalty it stands exactly ln(n) above
-    the rest's mean penalty-free level... kept simple: every key has value 0
-    but the needle (value 1 in channel 1); the weight the needle gets is
-    returned, to compare with the dense formula."""
+    """Every key scores 0 and has value 0, but the needle at key_pos: raw score
+    8, value 1 in channel 1. The output's channel 1 is then the softmax weight
+    the needle gets after the distance penalty; the caller compares it with
+    the dense formula. Pages are handed out in reverse order."""
     n = query_pos + 1
     nblocks = (n + block_size - 1) // block_size
     kc = torch.zeros(nblocks + 2, G, block_size, D, dtype=dtype)
