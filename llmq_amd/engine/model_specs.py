@@ -820,6 +820,299 @@ MUVETAR_PRESETS = {
 }
 
 
+# ---------------------------------------------------------------------------
+# Tefudra: a hybrid decoder on an fp32 residual whose norms work on equal
+# consecutive groups of the width. A layer carries either softmax attention
+# whose values are its keys (per-head q/k norm, partial rotation, a sliding
+# window that also keeps the first tokens, a learned extra term per head in
+# the softmax denominator), or two mixers side by side whose normed outputs
+# are averaged: tanh-capped sliding-window attention behind a short causal
+# convolution with position-rotated unit-norm values, and an mLSTM matrix
+# memory. Feed-forwards are dense (squared ReLU) or a softmax-routed mixture
+# of GELU experts with identity experts and a shared expert. A layer may run
+# on another layer's weights with a cache and state of its own.
+
+
+@dataclass
+class SinkAttnSpec:
+    """Softmax attention with grouped key/value heads whose values are the
+    keys as projected (before norm and rotation). Position i sees j <= i with
+    i - j < window (window 0: every j <= i) or j < keep_first; the softmax
+    denominator holds one more term exp(sink_head)."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    scale: float
+    rot: RotarySpec = None
+    window: int = 0
+    keep_first: int = 0
+    kind: str = "sink_attention"
+
+    @property
+    def vdim(self) -> int:
+        return self.dim
+
+
+@dataclass
+class CappedConvAttnSpec:
+    """Sliding-window softmax attention with biased projections, a causal
+    convolution of `conv` taps per channel on q, k and v, scores passed
+    through softcap * tanh(. / softcap) (softcap 0: none), values divided by
+    their root mean square per head and rotated by their own position over
+    all of vdim; a head's output is turned back by the query's position."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    rot: RotarySpec = None
+    window: int = 0
+    softcap: float = 0.0
+    conv: int = 1
+    kind: str = "capped_conv_attention"
+
+
+@dataclass
+class MLSTMSpec:
+    """Matrix memory per head with exponential gating: log input gate
+    i = cap tanh(. / cap), log forget gate f = logsigmoid(cap tanh(. / cap)),
+    running maximum m_t = max(f + m_(t-1), i) from m = 0,
+    S_t = e^(f + m_(t-1) - m_t) S_(t-1) + e^(i - m_t) k v^T, n_t alike with k,
+    o = S_t^T q / (max(|n_t . q|, e^(-m_t)) + 1e-6)."""
+
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+    kind: str = "mlstm"
+
+
+@dataclass
+class AveragedPairSpec:
+    """Two mixers on the same input; the result is half the sum of their
+    outputs, each RMS-normed over the model width with its own weight."""
+
+    left: CappedConvAttnSpec
+    right: MLSTMSpec
+    kind: str = "parallel"
+
+
+@dataclass
+class RoutedFFSpec:
+    """Mixture of ungated experts W_down gelu(W_up h) (exact GELU). Scores =
+    softmax of the router logits over experts + identity experts; the `top`
+    largest of score + correction are chosen, their scores divided by their
+    sum weigh the outputs; an identity expert returns its input. shared_ff >
+    0: one more expert of the same form runs for every token."""
+
+    experts: int
+    top: int
+    ff: int
+    identity: int = 0
+    shared_ff: int = 0
+
+
+@dataclass
+class TefudraLayerSpec:
+    mixer: object                           # SinkAttnSpec | AveragedPairSpec
+    ff: int = 0                             # dense feed-forward inner size (0 = none)
+    moe: Optional[RoutedFFSpec] = None
+    weights_of: Optional[int] = None        # runs on this layer's tensors
+
+
+@dataclass
+class TefudraSpec:
+    name: str
+    family: str                   # "tefudra"
+    vocab_size: int
+    hidden_size: int
+    layers: list = field(default_factory=list)
+    rms_eps: float = 1e-6
+    norm_groups: int = 1
+    max_position_embeddings: int = 1 << 17
+    tied_embeddings: bool = True
+    eos_token_id: int = 2
+    bos_token_id: int = 1
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    def owner(self, i: int) -> int:
+        """The layer whose tensors layer i runs on."""
+        seen = set()
+        while self.layers[i].weights_of is not None:
+            if i in seen:
+                raise ValueError("weights_of forms a cycle")
+            seen.add(i)
+            i = self.layers[i].weights_of
+        return i
+
+    def param_count(self) -> int:
+        w = self.hidden_size
+        total = self.vocab_size * w + w
+        for ls in self.layers:
+            if ls.weights_of is not None:
+                continue
+            m = ls.mixer
+            total += 4 * w if (ls.ff or ls.moe) else 2 * w
+            if m.kind == "sink_attention":
+                total += (m.heads + m.kv_heads) * m.dim * w + 2 * m.dim + m.heads
+                total += w * m.heads * m.dim
+            else:
+                a, r = m.left, m.right
+                n = a.heads * a.dim + a.kv_heads * (a.dim + a.vdim)
+                total += n * (w + 1 + a.conv) + w * a.heads * a.vdim + w
+                total += r.heads * (2 * r.dim + 2 * r.vdim) * w + r.heads * r.vdim
+                total += w * r.heads * r.vdim + 2 * r.heads * (w + 1) + 2 * w
+            if ls.ff:
+                total += 2 * w * ls.ff
+            if ls.moe:
+                e = ls.moe
+                total += (e.experts + e.identity) * (w + 1)
+                total += 2 * w * (e.experts * e.ff + e.shared_ff)
+        return total
+
+
+def _rotary_from(rc: dict, size: int, where: str) -> RotarySpec:
+    rot = RotarySpec(base=float(rc["base"]), dims=int(rc.get("dims", size)), layout="half")
+    if rot.dims % 2 or not 0 <= rot.dims <= size:
+        raise ValueError(f"{where}: rot.dims must be even and at most the head size")
+    return rot
+
+
+def tefudra_spec_from_config(cfg: dict, name: str) -> TefudraSpec:
+    """Tefudra config.json -> TefudraSpec: every size and constant comes from
+    the config."""
+    layers = []
+    raw = cfg["layers"]
+    for i, lc in enumerate(raw):
+        mc, kind = lc["mixer"], lc["type"]
+        if kind == "attention":
+            heads = int(mc["heads"])
+            mask = mc.get("mask") or {}
+            mixer = SinkAttnSpec(
+                heads=heads, kv_heads=int(mc.get("kv_heads", heads)), dim=int(mc["dim"]),
+                scale=float(mc.get("scale", int(mc["dim"]) ** -0.5)),
+                rot=_rotary_from(mc["rot"], int(mc["dim"]), f"layer {i}"),
+                window=int(mask.get("size", 0)), keep_first=int(mask.get("keep_first", 0)))
+            if int(mc.get("vdim", mixer.dim)) != mixer.dim:
+                raise ValueError(f"layer {i}: values are the keys, so vdim must equal dim")
+            pairs = [mixer]
+        elif kind == "parallel":
+            lt, rt = mc["left"], mc["right"]
+            heads = int(lt["heads"])
+            mask = lt.get("mask") or {}
+            left = CappedConvAttnSpec(
+                heads=heads, kv_heads=int(lt.get("kv_heads", heads)), dim=int(lt["dim"]),
+                vdim=int(lt.get("vdim", lt["dim"])),
+                scale=float(lt.get("scale", int(lt["dim"]) ** -0.5)),
+                rot=_rotary_from(lt["rot"], int(lt["dim"]), f"layer {i}"),
+                window=int(mask.get("size", 0)), softcap=float(lt.get("softcap") or 0.0),
+                conv=int(lt.get("conv", 1)))
+            if left.vdim % 2:
+                raise ValueError(f"layer {i}: rotated values need an even vdim")
+            if left.conv < 1:
+                raise ValueError(f"layer {i}: the convolution needs at least one tap")
+            right = MLSTMSpec(heads=int(rt["heads"]), dim=int(rt["dim"]), vdim=int(rt["vdim"]),
+                              gate_cap=float(rt["gate_cap"]))
+            mixer = AveragedPairSpec(left=left, right=right)
+            pairs = [left]
+        else:
+            raise ValueError(f"layer {i}: unknown mixer type {kind!r}")
+        for a in pairs:
+            if a.heads % a.kv_heads:
+                raise ValueError(f"layer {i}: heads must be a multiple of kv_heads")
+        mlp = lc.get("mlp")
+        ff, moe = 0, None
+        if mlp is not None:
+            if mlp.get("kind", "dense") == "dense":
+                ff = int(mlp["ff"])
+            elif mlp["kind"] == "moe":
+                rt, sh = mlp["router"], mlp.get("shared")
+                moe = RoutedFFSpec(experts=int(rt["experts"]), top=int(rt["top"]),
+                                   ff=int(mlp["expert"]["ff"]), identity=int(rt.get("identity", 0)),
+                                   shared_ff=int(sh["ff"]) if sh else 0)
+                if not 1 <= moe.top <= moe.experts + moe.identity:
+                    raise ValueError(f"layer {i}: top must be within 1..experts + identity")
+            else:
+                raise ValueError(f"layer {i}: unknown feed-forward kind {mlp['kind']!r}")
+        src = lc.get("weights_of")
+        if src is not None and not 0 <= int(src) < len(raw):
+            raise ValueError(f"layer {i}: weights_of names no layer")
+        layers.append(TefudraLayerSpec(mixer=mixer, ff=ff, moe=moe,
+                                       weights_of=None if src is None else int(src)))
+    spec = TefudraSpec(
+        name=name, family="tefudra", vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]), layers=layers, rms_eps=float(cfg["norm"]["eps"]),
+        norm_groups=int(cfg["norm"].get("groups", 1)))
+    if spec.hidden_size % spec.norm_groups:
+        raise ValueError("norm.groups must divide the width")
+    for i in range(len(layers)):
+        spec.owner(i)
+    return spec
+
+
+def _tefudra(name, vocab, width, n_layers, heads, kv_heads, dim, ff, window, keep_first=4,
+             groups=4, attn_every=3, left_dim=None, left_vdim=None, left_window=None, conv=4,
+             softcap=20.0, mem_heads=None, mem_dim=None, mem_vdim=None, gate_cap=15.0,
+             moe_every=0, experts=8, identity=2, top=2, expert_ff=None, shared_ff=0,
+             rot_dims=None, share_last=False, **kw):
+    """Preset builder: every `attn_every`-th layer is a sink-attention layer,
+    the others carry capped attention beside a matrix memory; every
+    `moe_every`-th feed-forward is a routed mixture, the others dense;
+    share_last: the last layer runs on the weights of the nearest earlier
+    layer of its kind."""
+    layers = []
+    ld, lv = left_dim or dim, left_vdim or left_dim or dim
+    for i in range(n_layers):
+        if attn_every and i % attn_every == attn_every - 1:
+            mixer = SinkAttnSpec(heads, kv_heads, dim, dim ** -0.5,
+                                 RotarySpec(1000000.0, rot_dims or dim, "half"), window, keep_first)
+        else:
+            mixer = AveragedPairSpec(
+                CappedConvAttnSpec(heads, kv_heads, ld, lv, ld ** -0.5,
+                                   RotarySpec(250000.0, ld, "half"), left_window or window,
+                                   softcap, conv),
+                MLSTMSpec(mem_heads or heads, mem_dim or dim, mem_vdim or dim, gate_cap))
+        if moe_every and i % moe_every == moe_every - 1:
+            layers.append(TefudraLayerSpec(mixer, moe=RoutedFFSpec(
+                experts, top, expert_ff or ff, identity, shared_ff)))
+        else:
+            layers.append(TefudraLayerSpec(mixer, ff=ff))
+    if share_last and n_layers > 1:
+        for j in range(n_layers - 2, -1, -1):
+            if layers[j].mixer.kind == layers[-1].mixer.kind:
+                layers[-1] = TefudraLayerSpec(layers[j].mixer, layers[j].ff, layers[j].moe, j)
+                break
+    return TefudraSpec(name=name, family="tefudra", vocab_size=vocab, hidden_size=width,
+                       layers=layers, norm_groups=groups, **kw)
+
+
+TEFUDRA_PRESETS = {
+    # CPU/GPU test config: both layer types, both feed-forwards, grouped kv
+    # heads, q/k size != v size, partial rotation, a shared-weights layer
+    "tiny-tefudra": _tefudra("tiny-tefudra", 512, 64, 6, 4, 2, 16, 96, 24, keep_first=3,
+                             groups=2, attn_every=3, left_dim=24, left_vdim=16, left_window=20,
+                             conv=3, softcap=8.0, mem_heads=2, mem_dim=8, mem_vdim=24,
+                             gate_cap=10.0, moe_every=2, experts=5, identity=2, top=3,
+                             expert_ff=32, shared_ff=48, rot_dims=8, share_last=True),
+    # benchmark configs at the layer sizes of llama-3.2-1b / -3b (and of the
+    # other hybrid presets): same width, head count, feed-forward and depth;
+    # every 4th layer sink attention, window 2048
+    "tefudra-1b": _tefudra("tefudra-1b", 128256, 2048, 16, 32, 8, 64, 8192, 2048, attn_every=4,
+                           mem_heads=16, mem_dim=64, mem_vdim=128),
+    "tefudra-1b-moe": _tefudra("tefudra-1b-moe", 128256, 2048, 16, 32, 8, 64, 8192, 2048,
+                               attn_every=4, mem_heads=16, mem_dim=64, mem_vdim=128,
+                               moe_every=2, experts=8, identity=2, top=2, expert_ff=2048,
+                               shared_ff=2048),
+    "tefudra-3b": _tefudra("tefudra-3b", 128256, 3072, 28, 24, 8, 128, 8192, 2048, attn_every=4,
+                           mem_heads=12, mem_dim=128, mem_vdim=256),
+}
+
+
 def spec_from_hf_config(path: Path, name: str) -> ModelSpec:
     """Build a spec from a HF checkpoint directory's config.json."""
     with open(path / "config.json", "r", encoding="utf-8") as fh:
@@ -828,6 +1121,8 @@ def spec_from_hf_config(path: Path, name: str) -> ModelSpec:
         return kosalorn_spec_from_config(cfg, name)
     if str(cfg.get("architecture", "")).lower() == "muvetar":
         return muvetar_spec_from_config(cfg, name)
+    if str(cfg.get("architecture", "")).lower() == "tefudra":
+        return tefudra_spec_from_config(cfg, name)
     if str(cfg.get("architecture", "")).lower() == "kakovik":
         st = path / "model.safetensors"
         return kakovik_spec_from_config(
@@ -909,7 +1204,9 @@ def resolve_spec(model: str) -> ModelSpec:
         return KOSALORN_PRESETS[key]
     if key in MUVETAR_PRESETS:
         return MUVETAR_PRESETS[key]
+    if key in TEFUDRA_PRESETS:
+        return TEFUDRA_PRESETS[key]
     raise ValueError(
         f"Unknown model '{model}'. Provide a checkpoint directory with config.json "
-        f"or one of: {sorted(PRESETS) + sorted(HYBRID_PRESETS) + sorted(KOSALORN_PRESETS) + sorted(MUVETAR_PRESETS) + sorted(ALIASES)}"
+        f"or one of: {sorted(PRESETS) + sorted(HYBRID_PRESETS) + sorted(KOSALORN_PRESETS) + sorted(MUVETAR_PRESETS) + sorted(TEFUDRA_PRESETS) + sorted(ALIASES)}"
     )

@@ -4,6 +4,7 @@ from llmq_amd.engine.models.kakovik import KakovikLM
 from llmq_amd.engine.models.kosalorn import KosalornLM
 from llmq_amd.engine.models.llama import CausalLM
 from llmq_amd.engine.models.muvetar import MuvetarLM
+from llmq_amd.engine.models.tefudra import TefudraLM
 
 MODEL_CLASSES = {
     "llama": CausalLM,
@@ -13,6 +14,7 @@ MODEL_CLASSES = {
     "kakovik": KakovikLM,
     "kosalorn": KosalornLM,
     "muvetar": MuvetarLM,
+    "tefudra": TefudraLM,
 }
 
 
@@ -23,4 +25,4 @@ def model_class_for(spec):
         raise ValueError(f"no model class registered for family {spec.family!r}") from None
 
 
-__all__ = ["CausalLM", "KakovikLM", "KosalornLM", "MuvetarLM", "MODEL_CLASSES", "model_class_for"]
+__all__ = ["CausalLM", "KakovikLM", "KosalornLM", "MuvetarLM", "TefudraLM", "MODEL_CLASSES", "model_class_for"]

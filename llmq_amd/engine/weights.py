@@ -344,5 +344,94 @@ def load_muvetar_weights(model, path: Path) -> None:
     logger.info("loaded %d tensors from %s", len(tensors), path)
 
 
+def load_tefudra_weights(model, path: Path) -> None:
+    """Tefudra checkpoint names -> the packed in-tree tensors.
+
+    Checkpoint: 'embed' (also the output head), 'final.norm', and per layer
+    that owns tensors 'l<i>.norm1', '.norm1b', '.norm2', '.norm2b', the mixer
+    under 'l<i>.mix.' (an averaged pair's two mixers under '.left.' and
+    '.right.', their output norms '.left.out' / '.right.out'), the
+    feed-forward under 'l<i>.mlp.' (experts 'e<j>.', the shared expert
+    'shared.'); linear weights are [out, in], a bias is the weight's name +
+    '.b', a short convolution's taps the weight's name + '.conv'. Packing:
+    everything that reads the mixer's input in the model dtype -> 'in' (+ the
+    biases -> 'in_b', the taps -> 'conv_w', segments at multiples of 8 rows),
+    the memory's input and forget gate rows -> one fp32 'gates', experts
+    stacked [E, ...]."""
+    tensors = _read_all(path)
+    used = set()
+
+    def get(name: str) -> torch.Tensor:
+        if name not in tensors:
+            raise KeyError(f"missing tensor {name}")
+        used.add(name)
+        return tensors[name]
+
+    def copy_(dst: torch.Tensor, src: torch.Tensor) -> None:
+        if dst.shape != src.shape:
+            raise ValueError(f"shape mismatch: {tuple(dst.shape)} vs {tuple(src.shape)}")
+        dst.copy_(src.to(dst.dtype))
+
+    copy_(model.embedding, get("embed"))
+    copy_(model.final_norm, get("final.norm"))
+    for i, ls, lw in model.owned_layers():
+        p, t, m = f"l{i}.", lw.t, ls.mixer
+        mx = p + "mix."
+        copy_(t["norm1"], get(p + "norm1"))
+        copy_(t["norm1b"], get(p + "norm1b"))
+
+        def put(seg: str, src: torch.Tensor, dst: str = "in", lw=lw, t=t) -> None:
+            at, n = lw.seg[seg]
+            copy_(t[dst][at:at + n], src)
+
+        t["in"].zero_()  # alignment rows between segments
+        if m.kind == "sink_attention":
+            put("q", get(mx + "q"))
+            put("k", get(mx + "k"))
+            copy_(t["q_norm"], get(mx + "q.norm"))
+            copy_(t["k_norm"], get(mx + "k.norm"))
+            copy_(t["sink"], get(mx + "sink"))
+            copy_(t["o"], get(mx + "o"))
+        else:
+            lf, rt = mx + "left.", mx + "right."
+            t["in_b"].zero_()
+            t["conv_w"].zero_()
+            for seg in ("q", "k", "v"):
+                put(seg, get(lf + seg))
+                put(seg, get(lf + seg + ".b"), "in_b")
+                put(seg, get(lf + seg + ".conv"), "conv_w")
+            copy_(t["o"], get(lf + "o"))
+            copy_(t["o_b"], get(lf + "o.b"))
+            copy_(t["left_out"], get(lf + "out"))
+            for seg, name in (("mq", "q"), ("mk", "k"), ("mv", "v"), ("mg", "g")):
+                put(seg, get(rt + name))
+            copy_(t["gates"], torch.cat([get(rt + "i"), get(rt + "f")], dim=0))
+            copy_(t["gates_b"], torch.cat([get(rt + "i.b"), get(rt + "f.b")], dim=0))
+            copy_(t["m_norm"], get(rt + "norm"))
+            copy_(t["m_o"], get(rt + "o"))
+            copy_(t["right_out"], get(rt + "out"))
+        if ls.ff or ls.moe:
+            copy_(t["norm2"], get(p + "norm2"))
+            copy_(t["norm2b"], get(p + "norm2b"))
+        if ls.ff:
+            copy_(t["up"], get(p + "mlp.up"))
+            copy_(t["down"], get(p + "mlp.down"))
+        if ls.moe:
+            e = ls.moe
+            copy_(t["router"], get(p + "mlp.router"))
+            copy_(t["correction"], get(p + "mlp.correction"))
+            for j in range(e.experts):
+                copy_(t["e_up"][j], get(f"{p}mlp.e{j}.up"))
+                copy_(t["e_down"][j], get(f"{p}mlp.e{j}.down"))
+            if e.shared_ff:
+                copy_(t["s_up"], get(p + "mlp.shared.up"))
+                copy_(t["s_down"], get(p + "mlp.shared.down"))
+    unused = sorted(set(tensors) - used)
+    if unused:
+        logger.warning("checkpoint tensors this configuration does not use: %s", unused[:8])
+    model.finalize()
+    logger.info("loaded %d tensors from %s", len(tensors), path)
+
+
 _FAMILY_LOADERS = {"kakovik": load_kakovik_weights, "kosalorn": load_kosalorn_weights,
-                   "muvetar": load_muvetar_weights}
+                   "muvetar": load_muvetar_weights, "tefudra": load_tefudra_weights}

@@ -401,23 +401,27 @@ def _use_hybrid(t: torch.Tensor) -> bool:
 
 
 def rmsnorm_cast(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float,
-                 out_dtype: torch.dtype) -> torch.Tensor:
-    """RMSNorm of x (fp32 stream or model dtype) written in out_dtype."""
+                 out_dtype: torch.dtype, groups: int = 1) -> torch.Tensor:
+    """RMSNorm of x (fp32 stream or model dtype) written in out_dtype.
+    groups > 1: every row is normed in that many equal consecutive parts,
+    each by its own root mean square."""
     if _use_hybrid(x):
         out = torch.empty(x.shape, dtype=out_dtype, device=x.device)
-        _HY.rmsnorm_cast(out, x, weight, eps, offset)
+        _HY.rmsnorm_cast(out, x, weight, eps, offset, int(groups))
         return out
-    return torch_ref.rmsnorm_cast(x, weight, eps, offset, out_dtype)
+    return torch_ref.rmsnorm_cast(x, weight, eps, offset, out_dtype, groups)
 
 
 def sandwich_norm_res32(x: torch.Tensor, residual: torch.Tensor, w_post: torch.Tensor,
-                        w_pre: torch.Tensor, eps: float, offset: float) -> torch.Tensor:
+                        w_pre: torch.Tensor, eps: float, offset: float,
+                        groups: int = 1) -> torch.Tensor:
     """residual (fp32, in place) += rmsnorm(x)·(w_post+offset); returns
-    rmsnorm(residual)·(w_pre+offset) in x's dtype (x's storage on GPU)."""
+    rmsnorm(residual)·(w_pre+offset) in x's dtype (x's storage on GPU).
+    groups > 1: both norms work on that many equal parts of a row."""
     if _use_hybrid(x):
-        _HY.sandwich_norm_res32(x, residual, w_post, w_pre, eps, offset)
+        _HY.sandwich_norm_res32(x, residual, w_post, w_pre, eps, offset, int(groups))
         return x
-    return torch_ref.sandwich_norm_res32(x, residual, w_post, w_pre, eps, offset)
+    return torch_ref.sandwich_norm_res32(x, residual, w_post, w_pre, eps, offset, groups)
 
 
 def act_and_mul(x: torch.Tensor, gelu: bool = False) -> torch.Tensor:
@@ -459,7 +463,7 @@ def chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables, cu_q,
         out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
         _HY.paged_attn_prefill(out, q, gate, k_cache, v_cache, bias, block_tables, cu_q,
                                q_start, int(max_q), int(span), float(scale), _MASK_BLOCK, 1,
-                               _BIAS_TABLE)
+                               _BIAS_TABLE, 0, None, 0.0)
         return out
     return torch_ref.chunk_bias_attn_prefill(q, gate, k_cache, v_cache, bias, block_tables,
                                              cu_q, q_start, span, scale)
@@ -471,7 +475,8 @@ def chunk_bias_attn_decode(q, gate, k_cache, v_cache, bias, block_tables, contex
     if _use_hybrid(q):
         out = torch.empty(q.shape[0], q.shape[1], v_cache.shape[3], dtype=q.dtype, device=q.device)
         _HY.paged_attn_decode(out, q, gate, k_cache, v_cache, bias, block_tables,
-                              context_lens, int(span), float(scale), _MASK_BLOCK, _BIAS_TABLE)
+                              context_lens, int(span), float(scale), _MASK_BLOCK, _BIAS_TABLE,
+                              0, None, 0.0)
         return out
     return torch_ref.chunk_bias_attn_decode(q, gate, k_cache, v_cache, bias, block_tables,
                                             context_lens, span, scale)
@@ -521,31 +526,38 @@ def head_norm(o, weight, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
 
 
 def window_attn_prefill(q, k_cache, v_cache, dv: int, block_tables, cu_q, q_start, max_q: int,
-                        window: int, scale: float, log_bias=None) -> torch.Tensor:
+                        window: int, scale: float, log_bias=None, keep_first: int = 0,
+                        sink=None, softcap: float = 0.0) -> torch.Tensor:
     """Softmax attention of packed prompt portions over the paged cache:
     query at position i sees keys j <= i with i - j < window (window 0:
-    every j <= i). v_cache None: the first dv channels of a key row are its
-    value (latent caches). log_bias fp32 [H, 2] = (r1, r2) per head: the
-    score loses r1 * ln(1 + r2 * (i - j)). q [T, H, D] -> [T, H, dv]."""
+    every j <= i) or j < keep_first. v_cache None: the first dv channels of a
+    key row are its value (latent caches). log_bias fp32 [H, 2] = (r1, r2)
+    per head: the score loses r1 * ln(1 + r2 * (i - j)). softcap c > 0: the
+    scaled score becomes c * tanh(score / c). sink fp32 [H]: the softmax
+    denominator gains exp(sink[h]). q [T, H, D] -> [T, H, dv]."""
     if _use_hybrid(q):
         out = torch.empty(q.shape[0], q.shape[1], dv, dtype=q.dtype, device=q.device)
         _HY.paged_attn_prefill(out, q, None, k_cache, v_cache, log_bias, block_tables, cu_q,
                                q_start, int(max_q), int(window) or _NO_WINDOW, float(scale),
-                               _MASK_WINDOW, 1, _BIAS_LOG if log_bias is not None else _BIAS_TABLE)
+                               _MASK_WINDOW, 1, _BIAS_LOG if log_bias is not None else _BIAS_TABLE,
+                               int(keep_first) if window else 0, sink, float(softcap))
         return out
     return torch_ref.window_attn_prefill(q, k_cache, v_cache, dv, block_tables, cu_q, q_start,
-                                         window, scale, log_bias)
+                                         window, scale, log_bias, keep_first, sink, softcap)
 
 
 def window_attn_decode(q, k_cache, v_cache, dv: int, block_tables, context_lens, window: int,
-                       scale: float, log_bias=None) -> torch.Tensor:
+                       scale: float, log_bias=None, keep_first: int = 0, sink=None,
+                       softcap: float = 0.0) -> torch.Tensor:
     """The single-token form: query b sits at position context_lens[b]-1."""
     if _use_hybrid(q):
         B, H, D = q.shape
         out = torch.empty(B, H, dv, dtype=q.dtype, device=q.device)
         bias_mode = _BIAS_LOG if log_bias is not None else _BIAS_TABLE
+        keep = int(keep_first) if window else 0
         if (q.dtype == torch.bfloat16 and k_cache.shape[1] == 1 and H >= 8 and D % 8 == 0
-                and D <= 256 and q.is_contiguous() and log_bias is None):
+                and D <= 256 and q.is_contiguous() and log_bias is None and not keep
+                and sink is None and not softcap):
             # one kv head for all query heads: the heads of a token become the
             # rows of one head, all at the token's position, and the step runs
             # on the matrix-core kernel — every key tile staged once for all
@@ -554,14 +566,14 @@ def window_attn_decode(q, k_cache, v_cache, dv: int, block_tables, context_lens,
             _HY.paged_attn_prefill(out.view(B * H, 1, dv), q.view(B * H, 1, D), None, k_cache,
                                    v_cache, None, block_tables, cu, context_lens - 1, H,
                                    int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW, 0,
-                                   _BIAS_TABLE)
+                                   _BIAS_TABLE, 0, None, 0.0)
             return out
         _HY.paged_attn_decode(out, q, None, k_cache, v_cache, log_bias, block_tables,
                               context_lens, int(window) or _NO_WINDOW, float(scale), _MASK_WINDOW,
-                              bias_mode)
+                              bias_mode, keep, sink, float(softcap))
         return out
     return torch_ref.window_attn_decode(q, k_cache, v_cache, dv, block_tables, context_lens,
-                                        window, scale, log_bias)
+                                        window, scale, log_bias, keep_first, sink, softcap)
 
 
 _HEAD_ROWS = {}
@@ -640,12 +652,15 @@ MOE_DENSE_MAX_PAIRS = 16384
 
 
 def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False, act: str = "silu",
-                limit: float = 0.0, weight_output: bool = False) -> torch.Tensor:
+                limit: float = 0.0, weight_output: bool = False, identity: int = 0) -> torch.Tensor:
     """Sum over a token's chosen experts of down_e(act(gate_e x, up_e x)).
     weight_output False: x = w * h (the router weight scales the expert's
     INPUT); True: x = h and the weight scales the expert's OUTPUT.
     act "silu": silu(g) * u; "clamp_swish": g * sigmoid(1.702 g) * (u + 1)
-    with g = min(g, limit), u = clamp(u, +-limit).
+    with g = min(g, limit), u = clamp(u, +-limit); "gelu_erf" / "relu2":
+    ungated experts down_e(act(up_e x)), gate_up then holds [E, F, W].
+    identity > 0 (with weight_output): indices E .. E + identity - 1 name
+    experts that return their input.
     h [T, W]; idx/w [T, top]; gate_up [E, 2F, W]; down [E, W, F].
 
     Few rows: one matrix-vector kernel pair that reads only each row's
@@ -656,45 +671,60 @@ def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False, act: str = "s
     and one GEMM pair per expert on contiguous slices (the per-expert row
     counts cross to the host once)."""
     T, top = idx.shape
-    act_mode = _MOE_ACTS[act]
+    gated = act in _MOE_ACTS
+    if identity and not weight_output:
+        raise ValueError("identity experts need the weight on the output side")
+    E = gate_up.shape[0]
+
+    def middle(gu):
+        if not gated:
+            return unary_act(gu, act)
+        return act_and_mul(gu) if act == "silu" else clamp_swish_mul(gu, limit)
+
     if h.is_cuda and (sync_free or T * top <= MOE_GEMV_MAX_ROWS):
         _use_hybrid(h)
         F_ = down.shape[2]
-        E = gate_up.shape[0]
-        if T * top >= MOE_GROUP_MIN_ROWS and E * T <= MOE_DENSE_MAX_PAIRS:
-            wd = torch.zeros(T, E, dtype=torch.float32, device=h.device)
+        plain = gated and not identity
+        if (T * top >= MOE_GROUP_MIN_ROWS and E * T <= MOE_DENSE_MAX_PAIRS) if plain \
+                else (sync_free or E * T <= MOE_DENSE_MAX_PAIRS):
+            wd = torch.zeros(T, E + identity, dtype=torch.float32, device=h.device)
             wd.scatter_(1, idx.long(), w)
             if weight_output:
                 xs = h.unsqueeze(0).expand(E, T, h.shape[1])
             else:  # zero input for the experts a token did not choose
                 xs = (h.float().unsqueeze(0) * wd.t().unsqueeze(-1)).to(h.dtype)
-            gu = torch.bmm(xs, gate_up.transpose(1, 2)).view(E * T, 2 * F_)
-            mid = act_and_mul(gu) if act == "silu" else clamp_swish_mul(gu, limit)
-            yk = torch.bmm(mid.view(E, T, F_), down.transpose(1, 2))
+            gu = torch.bmm(xs, gate_up.transpose(1, 2)).view(E * T, -1)
+            yk = torch.bmm(middle(gu).view(E, T, F_), down.transpose(1, 2))
             y = torch.empty_like(h)
+            if identity:
+                # an identity expert's output is the token itself: one more
+                # "expert result" whose weight is the sum of those chosen
+                yk = torch.cat([yk, h.unsqueeze(0)], dim=0)
+                wd = torch.cat([wd[:, :E], wd[:, E:].sum(dim=1, keepdim=True)], dim=1)
             _HY.moe_combine(y, yk, wd if weight_output else None)
             return y
-        hmid = torch.empty(T * top, F_, dtype=h.dtype, device=h.device)
-        w_in = None if weight_output else w
-        if MOE_GROUP_MIN_ROWS <= T * top <= MOE_GROUP_MAX_ROWS and \
-                max(h.shape[1], F_) * h.element_size() * 8 <= (128 << 10):
-            # enough rows that experts repeat: grouped by expert inside the
-            # kernel, a weight row is read once per 8 rows of its expert
-            _HY.moe_expert_gemv(hmid, h, idx, w_in, gate_up, True, act_mode, float(limit))
-            yk = torch.empty(T * top, h.shape[1], dtype=h.dtype, device=h.device)
-            _HY.moe_expert_gemv(yk, hmid, idx, None, down, False, 0, 0.0)
-            yk = yk.view(T, top, -1).float()
-            if weight_output:
-                yk = yk * w.unsqueeze(-1)
-            return yk.sum(dim=1).to(h.dtype)
-        _HY.moe_gate_up_gemv(hmid, h, idx, w_in, gate_up, act_mode, float(limit))
-        y = torch.empty_like(h)
-        _HY.moe_down_gemv(y, hmid, idx, down, w if weight_output else None)
-        return y
-    E = gate_up.shape[0]
+        if plain:
+            act_mode = _MOE_ACTS[act]
+            hmid = torch.empty(T * top, F_, dtype=h.dtype, device=h.device)
+            w_in = None if weight_output else w
+            if MOE_GROUP_MIN_ROWS <= T * top <= MOE_GROUP_MAX_ROWS and \
+                    max(h.shape[1], F_) * h.element_size() * 8 <= (128 << 10):
+                # enough rows that experts repeat: grouped by expert inside the
+                # kernel, a weight row is read once per 8 rows of its expert
+                _HY.moe_expert_gemv(hmid, h, idx, w_in, gate_up, True, act_mode, float(limit))
+                yk = torch.empty(T * top, h.shape[1], dtype=h.dtype, device=h.device)
+                _HY.moe_expert_gemv(yk, hmid, idx, None, down, False, 0, 0.0)
+                yk = yk.view(T, top, -1).float()
+                if weight_output:
+                    yk = yk * w.unsqueeze(-1)
+                return yk.sum(dim=1).to(h.dtype)
+            _HY.moe_gate_up_gemv(hmid, h, idx, w_in, gate_up, act_mode, float(limit))
+            y = torch.empty_like(h)
+            _HY.moe_down_gemv(y, hmid, idx, down, w if weight_output else None)
+            return y
     flat = idx.reshape(-1).long()
     order = torch.sort(flat, stable=True).indices
-    counts = torch.bincount(flat, minlength=E).tolist()
+    counts = torch.bincount(flat, minlength=E + identity).tolist()
     if weight_output:
         xs = h[order // top]
     else:
@@ -702,11 +732,12 @@ def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False, act: str = "s
     ys = torch.empty_like(xs)
     at = 0
     for e, n in enumerate(counts):
-        if n:
+        if n and e < E:
             gu = torch.nn.functional.linear(xs[at:at + n], gate_up[e])
-            mid = act_and_mul(gu) if act == "silu" else clamp_swish_mul(gu, limit)
-            ys[at:at + n] = torch.nn.functional.linear(mid, down[e])
-            at += n
+            ys[at:at + n] = torch.nn.functional.linear(middle(gu), down[e])
+        elif n:
+            ys[at:at + n] = xs[at:at + n]
+        at += n
     inv = torch.empty_like(order)
     inv[order] = torch.arange(order.numel(), device=order.device)
     if h.is_cuda:
@@ -783,14 +814,15 @@ def mingru_scan(z, u, g, z_b, u_b, state, cu, slots, fresh, out_dtype: torch.dty
     return torch_ref.mingru_scan(z, u, g, z_b, u_b, state, cu, slots, fresh, out_dtype)
 
 
-def causal_conv_silu(x, weight, bias, tail, cu, slots, fresh) -> torch.Tensor:
-    """Per-channel causal convolution + SiLU over packed sequences; tail
-    [slots, K-1, C] fp32 carries each sequence's last K-1 inputs."""
+def causal_conv_silu(x, weight, bias, tail, cu, slots, fresh, silu: bool = True) -> torch.Tensor:
+    """Per-channel causal convolution (+ bias unless None, + SiLU unless silu
+    is False) over packed sequences; tail [slots, K-1, C] fp32 carries each
+    sequence's last K-1 inputs."""
     if _use_hybrid(x):
         out = torch.empty(x.shape, dtype=x.dtype, device=x.device)
-        _HY.causal_conv_silu(out, x, weight, bias, tail, cu, slots, fresh)
+        _HY.causal_conv_silu(out, x, weight, bias, tail, cu, slots, fresh, bool(silu))
         return out
-    return torch_ref.causal_conv_silu(x, weight, bias, tail, cu, slots, fresh)
+    return torch_ref.causal_conv_silu(x, weight, bias, tail, cu, slots, fresh, silu)
 
 
 def selective_scan(x, dt, dt_b, A, Bm, Cm, D, z, state, cu, slots, fresh) -> torch.Tensor:
@@ -803,16 +835,18 @@ def selective_scan(x, dt, dt_b, A, Bm, Cm, D, z, state, cu, slots, fresh) -> tor
     return torch_ref.selective_scan(x, dt, dt_b, A, Bm, Cm, D, z, state, cu, slots, fresh)
 
 
-def softmax_topk(logits, top: int, scale: float = 1.0):
+def softmax_topk(logits, top: int, scale: float = 1.0, correction=None, renorm: bool = False):
     """Router: softmax over all experts in fp32, the `top` largest per row,
-    times scale: (indices int32 [T, top], weights fp32 [T, top])."""
+    times scale: (indices int32 [T, top], weights fp32 [T, top]). correction
+    fp32 [E]: the choice is made on score + correction, the weights stay the
+    plain scores. renorm: the chosen scores are divided by their sum first."""
     if _use_hybrid(logits):
         T = logits.shape[0]
         idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
         w = torch.empty(T, top, dtype=torch.float32, device=logits.device)
-        _HY.softmax_topk(idx, w, logits, int(top), float(scale))
+        _HY.softmax_topk(idx, w, logits, int(top), float(scale), correction, bool(renorm))
         return idx, w
-    return torch_ref.softmax_topk(logits, top, scale)
+    return torch_ref.softmax_topk(logits, top, scale, correction, renorm)
 
 
 def clamp_swish_mul(x, limit: float) -> torch.Tensor:
@@ -824,3 +858,93 @@ def clamp_swish_mul(x, limit: float) -> torch.Tensor:
         _HY.clamp_swish_mul(out, x, float(limit))
         return out
     return torch_ref.clamp_swish_mul(x, limit)
+
+
+# ---- windowed attention beside a matrix memory: norms on groups of the
+# width, kept first tokens and a learned softmax term, rotated values, mLSTM --
+
+
+def qkv_norm_rope_cache(q, k, v, q_w, k_w, inv_freq, rot_dims: int, positions, k_cache, v_cache,
+                        slots, eps: float, v_unit_norm: bool = False, v_inv_freq=None) -> None:
+    """Per token, between the projections and the attention kernel: optional
+    per-head RMSNorm of q and k (weights q_w / k_w [D]), rotary positions on
+    their first rot_dims channels (q [T, H, D] in place), and the paged-cache
+    scatter of k and of the values — v [T, G, DV], or the keys as they arrive
+    when v is None — which may be divided by their root mean square per head
+    (v_unit_norm) and turned by their position over all channels
+    (v_inv_freq fp32 [DV/2])."""
+    if _use_hybrid(q):
+        _HY.qkv_norm_rope_cache(q, k, v, q_w, k_w, inv_freq, int(rot_dims), positions, k_cache,
+                                v_cache, slots, float(eps), bool(v_unit_norm), v_inv_freq)
+        return
+    torch_ref.qkv_norm_rope_cache(q, k, v, q_w, k_w, inv_freq, rot_dims, positions, k_cache,
+                                  v_cache, slots, eps, v_unit_norm, v_inv_freq)
+
+
+def rotate_heads(x, positions, inv_freq, inverse: bool = False) -> torch.Tensor:
+    """x [T, H, n] in place: every head turned by its token's position (by
+    minus the position if inverse) over all n channels, pairs (i, i + n/2),
+    angles position * inv_freq[i] in fp32."""
+    if _use_hybrid(x):
+        _HY.rotate_heads(x, positions, inv_freq, bool(inverse))
+        return x
+    return torch_ref.rotate_heads(x, positions, inv_freq, inverse)
+
+
+def mlstm_gates(gates, cap: float, m_state, cu, slots, fresh):
+    """The gate recurrence of an mLSTM over packed sequences. gates fp32
+    [T, 2H] = input | forget pre-activations; returns fp32 [T, H] decay,
+    write and floor (see torch_ref.mlstm_gates); m_state [slots, H] fp32
+    (the running maximum) advanced in place."""
+    if _use_hybrid(gates):
+        T, H = gates.shape[0], gates.shape[1] // 2
+        out = torch.empty(3, T, H, dtype=torch.float32, device=gates.device)
+        _HY.mlstm_gates(out, gates, float(cap), m_state, cu, slots, fresh)
+        return out[0], out[1], out[2]
+    return torch_ref.mlstm_gates(gates, cap, m_state, cu, slots, fresh)
+
+
+def matrix_memory(q, k, v, decay, write, state, cu, slots, fresh, q_scale: float) -> torch.Tensor:
+    """mLSTM memory update and read-out with per-head scalar gates:
+    S <- decay S + write k [v | 1]^T, o = S^T (q_scale q). The state's last
+    value column is the normaliser vector, so o's last column is n . q.
+    state [slots, H, D, DV + 1] fp32 advanced in place; o [T, H, DV + 1] fp32."""
+    if _use_hybrid(q):
+        T, H, _ = q.shape
+        o = torch.empty(T, H, v.shape[2] + 1, dtype=torch.float32, device=q.device)
+        _HY.matrix_memory(o, q, k, v, decay, write, state, cu, slots, fresh, float(q_scale))
+        return o
+    return torch_ref.matrix_memory(q, k, v, decay, write, state, cu, slots, fresh, q_scale)
+
+
+def mlstm_out_norm_gate(o, floor, weight, gate, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """Read-out of an mLSTM: o[..., :DV] / (max(|o[..., DV]|, floor) + 1e-6),
+    per-head RMS norm, times weight [H*DV], times sigmoid(gate)."""
+    if _use_hybrid(o):
+        T, H, DV1 = o.shape
+        out = torch.empty(T, H * (DV1 - 1), dtype=out_dtype, device=o.device)
+        _HY.mlstm_out_norm_gate(out, o, floor, weight, gate, float(eps))
+        return out
+    return torch_ref.mlstm_out_norm_gate(o, floor, weight, gate, eps, out_dtype)
+
+
+def dual_norm_mean(a, w_a, b, w_b, eps: float) -> torch.Tensor:
+    """(rmsnorm(a) * w_a + rmsnorm(b) * w_b) / 2, norms over the whole row."""
+    if _use_hybrid(a):
+        out = torch.empty_like(a)
+        _HY.dual_norm_mean(out, a, w_a, b, w_b, float(eps))
+        return out
+    return torch_ref.dual_norm_mean(a, w_a, b, w_b, eps)
+
+
+_UNARY_ACTS = {"relu2": 0, "gelu_erf": 1}
+
+
+def unary_act(x, kind: str) -> torch.Tensor:
+    """Elementwise activation of an ungated feed-forward: "relu2" =
+    max(x, 0)^2, "gelu_erf" = the exact GELU."""
+    if _use_hybrid(x):
+        out = torch.empty_like(x)
+        _HY.unary_act(out, x, _UNARY_ACTS[kind])
+        return out
+    return torch_ref.unary_act(x, kind)

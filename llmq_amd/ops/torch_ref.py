@@ -248,17 +248,24 @@ def sample_tokens(
 
 
 def rmsnorm_cast(x: torch.Tensor, weight: torch.Tensor, eps: float, offset: float,
-                 out_dtype: torch.dtype) -> torch.Tensor:
+                 out_dtype: torch.dtype, groups: int = 1) -> torch.Tensor:
+    """groups > 1: the row is split into that many equal consecutive parts,
+    each divided by its own root mean square."""
     xf = x.float()
+    if groups > 1:
+        xf = xf.unflatten(-1, (groups, x.shape[-1] // groups))
     inv = 1.0 / torch.sqrt(xf.pow(2).mean(dim=-1, keepdim=True) + eps)
-    return (xf * inv * (weight.float() + offset)).to(out_dtype)
+    xf = xf * inv
+    if groups > 1:
+        xf = xf.flatten(-2)
+    return (xf * (weight.float() + offset)).to(out_dtype)
 
 
-def sandwich_norm_res32(x, residual, w_post, w_pre, eps, offset):
+def sandwich_norm_res32(x, residual, w_post, w_pre, eps, offset, groups=1):
     """residual(fp32) += rmsnorm(x)*(w_post+offset); returns
     rmsnorm(residual)*(w_pre+offset) in x's dtype. residual updated in place."""
-    residual.add_(rmsnorm_cast(x, w_post, eps, offset, torch.float32))
-    return rmsnorm_cast(residual, w_pre, eps, offset, x.dtype)
+    residual.add_(rmsnorm_cast(x, w_post, eps, offset, torch.float32, groups))
+    return rmsnorm_cast(residual, w_pre, eps, offset, x.dtype, groups)
 
 
 def act_and_mul(x: torch.Tensor, gelu: bool) -> torch.Tensor:
@@ -384,32 +391,42 @@ def gla_out_norm_gate(o, weight, gate, eps, out_dtype):
 # forget-gate recurrences, gated parallel residuals and expert mixtures.
 
 
-def _window_attend(qb, kc, vc, pos, window, scale, log_bias=None):
+def _window_attend(qb, kc, vc, pos, window, scale, log_bias=None, keep_first=0, sink=None,
+                   softcap=0.0):
     """qb [n, H, D] at absolute positions pos [n]; kc [L, G, D], vc [L, G, DV]
     cached keys/values of positions 0..L-1. Query i sees key j iff j <= i
-    and (window == 0 or i - j < window). log_bias [H, 2] = (r1, r2) per head
-    takes r1 * ln(1 + r2 * (i - j)) off the scaled score."""
+    and (window == 0 or i - j < window or j < keep_first). log_bias [H, 2] =
+    (r1, r2) per head takes r1 * ln(1 + r2 * (i - j)) off the scaled score.
+    softcap c > 0: the scaled score becomes c * tanh(score / c). sink [H]:
+    the softmax denominator gains exp(sink[h])."""
     n, H, _ = qb.shape
     G = kc.shape[1]
-    lo = max(0, int(pos[0]) - window + 1) if window else 0
+    lo = max(0, int(pos[0]) - window + 1) if window and not keep_first else 0
     kk = kc[lo:].float().repeat_interleave(H // G, dim=1)
     vv = vc[lo:].float().repeat_interleave(H // G, dim=1)
     j = torch.arange(lo, kc.shape[0], device=qb.device).view(1, -1)
     i = pos.view(-1, 1)
     vis = j <= i
     if window:
-        vis = vis & (i - j < window)
+        vis = vis & ((i - j < window) | (j < keep_first))
     scores = torch.einsum("ihd,jhd->hij", qb.float(), kk) * scale
+    if softcap:
+        scores = softcap * torch.tanh(scores / softcap)
     if log_bias is not None:
         dist = (i - j).clamp(min=0).float().unsqueeze(0)
         r1, r2 = log_bias[:, 0].float().view(-1, 1, 1), log_bias[:, 1].float().view(-1, 1, 1)
         scores = scores - r1 * torch.log1p(r2 * dist)
     scores = scores.masked_fill(~vis.unsqueeze(0), float("-inf"))
-    return torch.einsum("hij,jhd->ihd", torch.softmax(scores, dim=-1), vv)
+    if sink is not None:
+        extra = sink.float().view(-1, 1, 1).expand(H, n, 1)
+        w = torch.softmax(torch.cat([scores, extra], dim=-1), dim=-1)[..., :-1]
+    else:
+        w = torch.softmax(scores, dim=-1)
+    return torch.einsum("hij,jhd->ihd", w, vv)
 
 
 def window_attn_prefill(q, k_cache, v_cache, dv, block_tables, cu_q, q_start, window, scale,
-                        log_bias=None):
+                        log_bias=None, keep_first=0, sink=None, softcap=0.0):
     """Causal / sliding-window softmax attention of packed prompt portions
     over the paged cache. v_cache None: a key row's first dv channels are
     its value."""
@@ -424,12 +441,13 @@ def window_attn_prefill(q, k_cache, v_cache, dv, block_tables, cu_q, q_start, wi
         kc = _gather_seq(k_cache, block_tables[b], L)
         vc = kc[..., :dv] if v_cache is None else _gather_seq(v_cache, block_tables[b], L)
         pos = torch.arange(p0, L, device=q.device)
-        out[s:e] = _window_attend(q[s:e], kc, vc, pos, window, scale, log_bias).to(q.dtype)
+        out[s:e] = _window_attend(q[s:e], kc, vc, pos, window, scale, log_bias, keep_first,
+                                  sink, softcap).to(q.dtype)
     return out
 
 
 def window_attn_decode(q, k_cache, v_cache, dv, block_tables, context_lens, window, scale,
-                       log_bias=None):
+                       log_bias=None, keep_first=0, sink=None, softcap=0.0):
     B, H, _ = q.shape
     out = q.new_empty(B, H, dv)
     for b in range(B):
@@ -438,7 +456,7 @@ def window_attn_decode(q, k_cache, v_cache, dv, block_tables, context_lens, wind
         vc = kc[..., :dv] if v_cache is None else _gather_seq(v_cache, block_tables[b], L)
         pos = torch.tensor([L - 1], device=q.device)
         out[b : b + 1] = _window_attend(q[b : b + 1], kc, vc, pos, window, scale,
-                                        log_bias).to(q.dtype)
+                                        log_bias, keep_first, sink, softcap).to(q.dtype)
     return out
 
 
@@ -618,8 +636,9 @@ def mingru_scan(z, u, g, z_b, u_b, state, cu, slots, fresh, out_dtype):
     return (out * torch.nn.functional.silu(g.float())).to(out_dtype)
 
 
-def causal_conv_silu(x, weight, bias, tail, cu, slots, fresh):
-    """Per-channel causal convolution + SiLU over packed sequences.
+def causal_conv_silu(x, weight, bias, tail, cu, slots, fresh, silu=True):
+    """Per-channel causal convolution (+ SiLU unless silu is False; bias may
+    be None) over packed sequences.
     x [T, C]; weight [C, K] fp32 (last column = the current token's tap);
     bias [C] fp32; tail [slots, K-1, C] fp32 holds each sequence's last K-1
     inputs (zeros before the start), advanced in place. Returns [T, C] in
@@ -633,13 +652,15 @@ def causal_conv_silu(x, weight, bias, tail, cu, slots, fresh):
         past = torch.zeros_like(tail[slot]) if int(fresh[b]) else tail[slot].clone()
         seq = torch.cat([past, xf[s:e]], dim=0)          # [K-1 + n, C]
         n = e - s
-        acc = bias.float().unsqueeze(0).expand(n, -1).clone()
+        acc = torch.zeros(n, x.shape[1], dtype=torch.float32, device=x.device)
+        if bias is not None:
+            acc += bias.float()
         for k in range(K):
             acc += seq[k:k + n] * weight[:, k].float()
         out[s:e] = acc
         if K > 1:
             tail[slot] = seq[seq.shape[0] - (K - 1):]
-    return torch.nn.functional.silu(out).to(x.dtype)
+    return (torch.nn.functional.silu(out) if silu else out).to(x.dtype)
 
 
 def selective_scan(x, dt, dt_b, A, Bm, Cm, D, z, state, cu, slots, fresh):
@@ -662,11 +683,20 @@ def selective_scan(x, dt, dt_b, A, Bm, Cm, D, z, state, cu, slots, fresh):
     return (y * torch.nn.functional.silu(z.float())).to(x.dtype)
 
 
-def softmax_topk(logits, top, scale):
+def softmax_topk(logits, top, scale, correction=None, renorm=False):
     """Router: scores = softmax(logits) over all experts (fp32); the `top`
-    largest per row, times scale. Returns (indices int32, weights fp32)."""
+    largest per row, times scale. correction [E]: the choice is made on
+    score + correction, the weights stay the plain scores. renorm: the chosen
+    scores are divided by their sum (+ 1e-20) first. Returns (indices int32,
+    weights fp32)."""
     s = torch.softmax(logits.float(), dim=-1)
-    w, idx = torch.topk(s, top, dim=-1)
+    if correction is None:
+        w, idx = torch.topk(s, top, dim=-1)
+    else:
+        idx = torch.topk(s + correction.float(), top, dim=-1).indices
+        w = torch.gather(s, 1, idx)
+    if renorm:
+        w = w / (w.sum(dim=-1, keepdim=True) + 1e-20)
     return idx.to(torch.int32), w * scale
 
 
@@ -681,3 +711,133 @@ def clamp_swish_mul(x, limit):
 
 def softcap(x, cap):
     return cap * torch.tanh(x.float() / cap)
+
+
+# --------------------------- windowed attention beside a matrix memory (ref) --
+# Reference forms of the ops added for decoders whose norms work on groups of
+# the width, whose attention keeps its first tokens and a learned term in the
+# softmax denominator or rotates its values, and whose recurrent mixer is an
+# mLSTM matrix memory.
+
+
+def qkv_norm_rope_cache(q, k, v, q_w, k_w, inv_freq, rot_dims, positions, k_cache, v_cache,
+                        slots, eps, v_unit_norm, v_inv_freq):
+    """Per token, between the projections and the attention kernel. q [T, H, D]
+    (updated in place), k [T, G, D], v [T, G, DV] or None (the values are then
+    the keys as they arrive). q_w / k_w [D] or None: per-head RMSNorm with that
+    weight first. Rotary positions (fp32 angle position * inv_freq[i], pairs
+    (i, i + rot_dims/2)) on the first rot_dims channels of q and k.
+    v_unit_norm: each head's value divided by its root mean square;
+    v_inv_freq [DV/2]: the value turned by its position over all DV channels.
+    k and v go to the paged cache rows `slots` (negative: skipped)."""
+    T, H, D = q.shape
+    G = k.shape[1]
+    raw_k = k.float()
+    qf, kf = q.float(), raw_k
+    if q_w is not None:
+        qf = qf / torch.sqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * q_w.float()
+    if k_w is not None:
+        kf = kf / torch.sqrt(kf.pow(2).mean(-1, keepdim=True) + eps) * k_w.float()
+    if rot_dims:
+        qf = _rotate(qf, positions, inv_freq, rot_dims, False)
+        kf = _rotate(kf, positions, inv_freq, rot_dims, False)
+    vf = raw_k if v is None else v.float()
+    if v_unit_norm:
+        vf = vf / torch.sqrt(vf.pow(2).mean(-1, keepdim=True) + eps)
+    if v_inv_freq is not None:
+        vf = _rotate(vf, positions, v_inv_freq, vf.shape[-1], False)
+    q.copy_(qf.to(q.dtype))
+    bs = k_cache.shape[2]
+    keep = slots >= 0
+    s = slots[keep].long()
+    k_cache[s // bs, :, s % bs, :] = kf[keep].to(k_cache.dtype)
+    v_cache[s // bs, :, s % bs, :] = vf[keep].to(v_cache.dtype)
+
+
+def rotate_heads(x, positions, inv_freq, inverse):
+    """x [T, H, n] in place: every head turned by (minus, if inverse) its
+    token's position over all n channels, pairs (i, i + n/2)."""
+    ang = inv_freq if not inverse else -inv_freq
+    x.copy_(_rotate(x.float(), positions, ang, x.shape[-1], False).to(x.dtype))
+    return x
+
+
+def mlstm_gates(gates, cap, m_state, cu, slots, fresh):
+    """gates [T, 2H] fp32 = (input | forget) pre-activations. Per head:
+    i = cap tanh(g_i / cap), f = logsigmoid(cap tanh(g_f / cap)),
+    m_t = max(f + m_(t-1), i) with m = 0 before a sequence's first token.
+    Returns fp32 [T, H] each: decay e^(f + m_(t-1) - m_t), write e^(i - m_t),
+    floor e^(-m_t); m_state [slots, H] advanced in place."""
+    T, H2 = gates.shape
+    H = H2 // 2
+    gi = cap * torch.tanh(gates[:, :H].float() / cap)
+    gf = torch.nn.functional.logsigmoid(cap * torch.tanh(gates[:, H:].float() / cap))
+    decay = torch.empty(T, H, dtype=torch.float32, device=gates.device)
+    write, floor = torch.empty_like(decay), torch.empty_like(decay)
+    for b in range(len(slots)):
+        s, e = int(cu[b]), int(cu[b + 1])
+        slot = int(slots[b])
+        m = torch.zeros(H, dtype=torch.float32, device=gates.device) if int(fresh[b]) \
+            else m_state[slot].clone()
+        for t in range(s, e):
+            new = torch.maximum(gf[t] + m, gi[t])
+            decay[t] = torch.exp(gf[t] + m - new)
+            write[t] = torch.exp(gi[t] - new)
+            floor[t] = torch.exp(-new)
+            m = new
+        m_state[slot] = m
+    return decay, write, floor
+
+
+def matrix_memory(q, k, v, decay, write, state, cu, slots, fresh, q_scale):
+    """S <- decay S + write k v'^T per head over packed sequences with
+    v' = [v | 1] (the last column carries the normaliser), o = S^T (q_scale q).
+    q, k [T, H, D], v [T, H, DV], decay / write [T, H] fp32; state
+    [slots, H, D, DV + 1] fp32 advanced in place. Returns o [T, H, DV + 1]."""
+    T, H, D = q.shape
+    DV = v.shape[2]
+    o = torch.empty(T, H, DV + 1, dtype=torch.float32, device=q.device)
+    qf = q.float() * q_scale
+    kf = k.float() * write.unsqueeze(-1)
+    vf = torch.cat([v.float(), torch.ones(T, H, 1, device=q.device)], dim=-1)
+    for b in range(len(slots)):
+        s, e = int(cu[b]), int(cu[b + 1])
+        slot = int(slots[b])
+        S = torch.zeros_like(state[slot]) if int(fresh[b]) else state[slot].clone()
+        for t in range(s, e):
+            S = decay[t].view(H, 1, 1) * S + kf[t].unsqueeze(-1) * vf[t].unsqueeze(-2)
+            o[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[slot] = S
+    return o
+
+
+def mlstm_out_norm_gate(o, floor, weight, gate, eps, out_dtype):
+    """o [T, H, DV + 1] (last column n . q), floor [T, H]: each head's
+    o[..., :DV] / (max(|n . q|, floor) + 1e-6), divided by its root mean
+    square, times weight [H * DV], times sigmoid(gate [T, H * DV])."""
+    T, H, DV1 = o.shape
+    DV = DV1 - 1
+    den = torch.maximum(o[..., DV].abs(), floor) + 1e-6
+    y = o[..., :DV] / den.unsqueeze(-1)
+    y = y / torch.sqrt(y.pow(2).mean(dim=-1, keepdim=True) + eps)
+    y = y.reshape(T, H * DV) * weight.float() * torch.sigmoid(gate.float())
+    return y.to(out_dtype)
+
+
+def dual_norm_mean(a, w_a, b, w_b, eps):
+    """(rmsnorm(a) * w_a + rmsnorm(b) * w_b) / 2 in a's dtype."""
+    ya = rmsnorm_cast(a, w_a, eps, 0.0, torch.float32)
+    yb = rmsnorm_cast(b, w_b, eps, 0.0, torch.float32)
+    return (0.5 * (ya + yb)).to(a.dtype)
+
+
+def unary_act(x, kind):
+    """relu2: max(x, 0)^2; gelu_erf: the exact GELU."""
+    xf = x.float()
+    if kind == "relu2":
+        y = torch.relu(xf).pow(2)
+    elif kind == "gelu_erf":
+        y = torch.nn.functional.gelu(xf)
+    else:
+        raise ValueError(f"unknown activation {kind!r}")
+    return y.to(x.dtype)
