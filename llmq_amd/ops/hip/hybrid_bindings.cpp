@@ -32,43 +32,52 @@ void allow_lds(K kernel, size_t bytes) {
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes));
 }
 
-void rmsnorm_cast(at::Tensor out, at::Tensor in, at::Tensor weight, double eps, double offset) {
+void rmsnorm_cast(at::Tensor out, at::Tensor in, at::Tensor weight, double eps, double offset,
+                  int64_t groups_arg) {
   HY_GPU(in);
   // in: contiguous, or 2-D rows with a stride (a column slice of a wider matrix)
   TORCH_CHECK(out.is_contiguous() && weight.is_contiguous());
   TORCH_CHECK(in.is_contiguous() || (in.dim() == 2 && in.stride(1) == 1),
               "rmsnorm_cast: in must be contiguous or row-strided 2-D");
-  const int hidden = in.size(-1);
-  TORCH_CHECK(out.sizes() == in.sizes() && weight.numel() == hidden);
+  const int width = in.size(-1);
+  TORCH_CHECK(out.sizes() == in.sizes() && weight.numel() == width);
   TORCH_CHECK(weight.scalar_type() == out.scalar_type(), "weight dtype must equal out dtype");
+  const int groups = (int)groups_arg;
+  TORCH_CHECK(groups >= 1 && width % groups == 0, "groups must divide the row");
+  // a row normed in groups is `groups` rows of width / groups to the kernel
+  const int hidden = width / groups;
   const long rows = in.numel() / hidden;
   if (rows == 0) return;
-  const long in_stride = in.is_contiguous() ? hidden : in.stride(0);
+  const long in_stride = in.is_contiguous() ? width : in.stride(0);
   hy_dispatch(out, "rmsnorm_cast", [&]<typename TO>() {
     if (in.scalar_type() == at::kFloat) {
       hipLaunchKernelGGL((rmsnorm_cast_kernel<float, TO>), dim3(rows), dim3(256), 0, hy_stream(),
                          reinterpret_cast<TO*>(out.data_ptr()), in.data_ptr<float>(), in_stride,
                          reinterpret_cast<const TO*>(weight.data_ptr()), hidden, (float)eps,
-                         (float)offset);
+                         (float)offset, groups);
     } else {
       TORCH_CHECK(in.scalar_type() == out.scalar_type(), "rmsnorm_cast: in must be fp32 or out's dtype");
       hipLaunchKernelGGL((rmsnorm_cast_kernel<TO, TO>), dim3(rows), dim3(256), 0, hy_stream(),
                          reinterpret_cast<TO*>(out.data_ptr()),
                          reinterpret_cast<const TO*>(in.data_ptr()), in_stride,
                          reinterpret_cast<const TO*>(weight.data_ptr()), hidden, (float)eps,
-                         (float)offset);
+                         (float)offset, groups);
     }
   });
 }
 
 void sandwich_norm_res32(at::Tensor x, at::Tensor residual, at::Tensor w_post, at::Tensor w_pre,
-                         double eps, double offset) {
+                         double eps, double offset, int64_t groups_arg) {
   HY_GPU(x);
   TORCH_CHECK(x.is_contiguous() && residual.is_contiguous());
   TORCH_CHECK(residual.scalar_type() == at::kFloat, "residual must be fp32");
-  const int hidden = x.size(-1);
-  TORCH_CHECK(residual.sizes() == x.sizes() && w_post.numel() == hidden && w_pre.numel() == hidden);
+  const int width = x.size(-1);
+  TORCH_CHECK(residual.sizes() == x.sizes() && w_post.numel() == width && w_pre.numel() == width);
   TORCH_CHECK(w_post.scalar_type() == x.scalar_type() && w_pre.scalar_type() == x.scalar_type());
+  TORCH_CHECK(w_post.is_contiguous() && w_pre.is_contiguous());
+  const int groups = (int)groups_arg;
+  TORCH_CHECK(groups >= 1 && width % groups == 0, "groups must divide the row");
+  const int hidden = width / groups;
   const long rows = x.numel() / hidden;
   if (rows == 0) return;
   if (x.scalar_type() == at::kBFloat16 && hidden % 8 == 0 && hidden <= 4 * 2048) {
@@ -78,7 +87,7 @@ void sandwich_norm_res32(at::Tensor x, at::Tensor residual, at::Tensor w_post, a
                          reinterpret_cast<bf*>(x.data_ptr()), residual.data_ptr<float>(),
                          reinterpret_cast<const bf*>(w_post.data_ptr()),
                          reinterpret_cast<const bf*>(w_pre.data_ptr()), hidden, (float)eps,
-                         (float)offset);
+                         (float)offset, groups);
     };
     if (hidden <= 2048) launch.template operator()<1>();
     else if (hidden <= 4096) launch.template operator()<2>();
@@ -90,7 +99,7 @@ void sandwich_norm_res32(at::Tensor x, at::Tensor residual, at::Tensor w_post, a
                        reinterpret_cast<T*>(x.data_ptr()), residual.data_ptr<float>(),
                        reinterpret_cast<const T*>(w_post.data_ptr()),
                        reinterpret_cast<const T*>(w_pre.data_ptr()), hidden, (float)eps,
-                       (float)offset);
+                       (float)offset, groups);
   });
 }
 
@@ -219,6 +228,14 @@ AttnDims attn_check(const at::Tensor& out, const at::Tensor& q, const std::optio
   return a;
 }
 
+// the learned softmax term per query head: fp32 [H], or none
+const float* sink_check(const std::optional<at::Tensor>& sink, const at::Tensor& q) {
+  if (!sink.has_value()) return nullptr;
+  TORCH_CHECK(sink->is_cuda() && sink->scalar_type() == at::kFloat && sink->is_contiguous() &&
+              sink->numel() == q.size(1), "sink must be fp32 [H] on the GPU");
+  return sink->data_ptr<float>();
+}
+
 template <typename F>
 void dispatch_nv(int DV, F&& f) {
   if (DV <= 64) f.template operator()<1>();
@@ -231,8 +248,14 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
                         at::Tensor k_cache, const std::optional<at::Tensor>& v_cache,
                         const std::optional<at::Tensor>& bias, at::Tensor block_tables,
                         at::Tensor cu_q, at::Tensor q_start, int64_t max_q, int64_t span,
-                        double scale, int64_t mask_mode, int64_t pos_stride, int64_t bias_mode) {
+                        double scale, int64_t mask_mode, int64_t pos_stride, int64_t bias_mode,
+                        int64_t keep_first, const std::optional<at::Tensor>& sink, double softcap) {
   if (q.size(0) == 0) return;
+  const float* sink_ptr = sink_check(sink, q);
+  TORCH_CHECK(keep_first >= 0 && softcap >= 0.0);
+  TORCH_CHECK(keep_first == 0 || mask_mode == kMaskWindow, "kept first tokens go with the window mask");
+  TORCH_CHECK(pos_stride == 1 || (keep_first == 0 && !sink_ptr),
+              "rows that share a position take no kept tokens and no sink");
   TORCH_CHECK(pos_stride == 0 || pos_stride == 1, "pos_stride is 0 (rows share a position) or 1");
   const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span, mask_mode,
                                 bias_mode);
@@ -282,7 +305,8 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
                          (int)span, (float)scale, a.v_row, (int)mask_mode, (int)pos_stride,
-                         n_split, n_split > 1 ? part.data_ptr<float>() : nullptr, (int)bias_mode);
+                         n_split, n_split > 1 ? part.data_ptr<float>() : nullptr, (int)bias_mode,
+                         (int)keep_first, sink_ptr, (float)softcap);
     };
     if (ksn <= 2 && dtn <= 4) launch.template operator()<2, 4>();
     else if (ksn <= 4 && dtn <= 8) launch.template operator()<4, 8>();
@@ -313,7 +337,8 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
                          reinterpret_cast<const T*>(a.vptr), a.bias, a.bias_len,
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          cu_q.data_ptr<int>(), q_start.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs,
-                         (int)span, (float)scale, a.v_row, (int)mask_mode, (int)bias_mode);
+                         (int)span, (float)scale, a.v_row, (int)mask_mode, (int)bias_mode,
+                         (int)keep_first, sink_ptr, (float)softcap);
     });
   });
 }
@@ -322,8 +347,12 @@ void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Ten
                        at::Tensor k_cache, const std::optional<at::Tensor>& v_cache,
                        const std::optional<at::Tensor>& bias, at::Tensor block_tables,
                        at::Tensor context_lens, int64_t span, double scale, int64_t mask_mode,
-                       int64_t bias_mode) {
+                       int64_t bias_mode, int64_t keep_first, const std::optional<at::Tensor>& sink,
+                       double softcap) {
   if (q.size(0) == 0) return;
+  const float* sink_ptr = sink_check(sink, q);
+  TORCH_CHECK(keep_first >= 0 && softcap >= 0.0);
+  TORCH_CHECK(keep_first == 0 || mask_mode == kMaskWindow, "kept first tokens go with the window mask");
   const AttnDims a = attn_check(out, q, gate, k_cache, v_cache, bias, block_tables, span, mask_mode,
                                 bias_mode);
   HY_I32(context_lens);
@@ -352,7 +381,8 @@ void paged_attn_decode(at::Tensor out, at::Tensor q, const std::optional<at::Ten
                          reinterpret_cast<const T*>(a.vptr), a.bias, a.bias_len,
                          block_tables.data_ptr<int>(), (int)block_tables.stride(0),
                          context_lens.data_ptr<int>(), a.H, a.G, a.D, a.DV, a.bs, (int)span,
-                         (float)scale, a.v_row, (int)mask_mode, (int)bias_mode);
+                         (float)scale, a.v_row, (int)mask_mode, (int)bias_mode, (int)keep_first,
+                         sink_ptr, (float)softcap);
       };
       if (hpw == 8) launch.template operator()<8>();
       else if (hpw == 4) launch.template operator()<4>();
@@ -414,7 +444,8 @@ void gla_recurrence(at::Tensor o, at::Tensor q, const std::optional<at::Tensor>&
                          reinterpret_cast<const T*>(z.data_ptr()), z.stride(0),
                          z_bias.data_ptr<float>(), state.data_ptr<float>(), cu.data_ptr<int>(),
                          slots.data_ptr<int>(), fresh.data_ptr<int>(), H, D, DV,
-                         (float)(1.0 / tau), q_scale, lower_ptr, (int)q_silu);
+                         (float)(1.0 / tau), q_scale, lower_ptr, (int)q_silu,
+                         static_cast<const float*>(nullptr), static_cast<const float*>(nullptr), 0);
     };
     if (D <= 32) launch.template operator()<2>();
     else if (D <= 64) launch.template operator()<4>();
@@ -920,16 +951,24 @@ void mingru_scan(at::Tensor out, at::Tensor z, at::Tensor u, at::Tensor g, at::T
 }
 
 // x [T, C] row-strided; weight [C, K] fp32; tail [slots, K-1, C] fp32.
-void causal_conv_silu(at::Tensor out, at::Tensor x, at::Tensor weight, at::Tensor bias,
-                      at::Tensor tail, at::Tensor cu, at::Tensor slots, at::Tensor fresh) {
+void causal_conv_silu(at::Tensor out, at::Tensor x, at::Tensor weight,
+                      const std::optional<at::Tensor>& bias_opt, at::Tensor tail, at::Tensor cu,
+                      at::Tensor slots, at::Tensor fresh, bool silu) {
   HY_GPU(x);
   HY_INNER(x);
   TORCH_CHECK(x.dim() == 2);
   const long T_ = x.size(0);
   const int C = x.size(1);
   if (T_ == 0) return;
-  HY_F32(weight); HY_F32(bias);
-  TORCH_CHECK(weight.dim() == 2 && weight.size(0) == C && bias.numel() == C);
+  HY_F32(weight);
+  TORCH_CHECK(weight.dim() == 2 && weight.size(0) == C);
+  const float* bias_ptr = nullptr;
+  if (bias_opt.has_value()) {
+    const at::Tensor& bias = *bias_opt;
+    HY_F32(bias);
+    TORCH_CHECK(bias.numel() == C);
+    bias_ptr = bias.data_ptr<float>();
+  }
   const int K = weight.size(1);
   TORCH_CHECK(K >= 1 && K <= kConvMaxTaps, "1 to ", kConvMaxTaps, " taps");
   TORCH_CHECK(out.is_contiguous() && out.sizes() == x.sizes() && out.scalar_type() == x.scalar_type());
@@ -941,9 +980,9 @@ void causal_conv_silu(at::Tensor out, at::Tensor x, at::Tensor weight, at::Tenso
   hy_dispatch(x, "causal_conv_silu", [&]<typename T>() {
     hipLaunchKernelGGL(causal_conv_silu_kernel<T>, grid, dim3(256), 0, hy_stream(),
                        reinterpret_cast<T*>(out.data_ptr()), reinterpret_cast<const T*>(x.data_ptr()),
-                       x.stride(0), weight.data_ptr<float>(), bias.data_ptr<float>(),
+                       x.stride(0), weight.data_ptr<float>(), bias_ptr,
                        tail.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(),
-                       fresh.data_ptr<int>(), d.B, C, K, rpt);
+                       fresh.data_ptr<int>(), d.B, C, K, rpt, (int)silu);
     if (K > 1)
       hipLaunchKernelGGL(conv_tail_update_kernel<T>, dim3((C + 255) / 256, d.B), dim3(256), 0,
                          hy_stream(), reinterpret_cast<const T*>(x.data_ptr()), x.stride(0),
@@ -1013,7 +1052,8 @@ void selective_scan(at::Tensor out, at::Tensor x, at::Tensor dt, at::Tensor dt_b
   });
 }
 
-void softmax_topk(at::Tensor idx, at::Tensor w, at::Tensor logits, int64_t top, double scale) {
+void softmax_topk(at::Tensor idx, at::Tensor w, at::Tensor logits, int64_t top, double scale,
+                  const std::optional<at::Tensor>& correction, bool renorm) {
   HY_GPU(logits);
   TORCH_CHECK(logits.dim() == 2 && logits.is_contiguous() && logits.scalar_type() == at::kFloat,
               "router logits must be fp32 [T, E]");
@@ -1024,9 +1064,15 @@ void softmax_topk(at::Tensor idx, at::Tensor w, at::Tensor logits, int64_t top, 
   HY_I32(idx);
   TORCH_CHECK(idx.dim() == 2 && idx.size(0) == rows && idx.size(1) == top);
   TORCH_CHECK(w.scalar_type() == at::kFloat && w.is_contiguous() && w.sizes() == idx.sizes());
+  const float* corr = nullptr;
+  if (correction.has_value()) {
+    TORCH_CHECK(correction->is_cuda() && correction->scalar_type() == at::kFloat &&
+                correction->is_contiguous() && correction->numel() == E, "correction must be fp32 [E]");
+    corr = correction->data_ptr<float>();
+  }
   hipLaunchKernelGGL(softmax_topk_kernel, dim3((rows + 3) / 4), dim3(256), 0, hy_stream(),
                      idx.data_ptr<int>(), w.data_ptr<float>(), logits.data_ptr<float>(), rows, E,
-                     (int)top, (float)scale);
+                     (int)top, (float)scale, corr, (int)renorm);
 }
 
 void clamp_swish_mul(at::Tensor out, at::Tensor in, double limit) {
@@ -1053,15 +1099,237 @@ void clamp_swish_mul(at::Tensor out, at::Tensor in, double limit) {
   });
 }
 
+// ---- windowed attention beside a matrix memory -------------------------------
+
+// q [T, H, D], k [T, G, D], v [T, G, DV] or none: row-strided views with packed heads.
+void qkv_norm_rope_cache(at::Tensor q, at::Tensor k, const std::optional<at::Tensor>& v_opt,
+                         const std::optional<at::Tensor>& q_w, const std::optional<at::Tensor>& k_w,
+                         const std::optional<at::Tensor>& inv_freq, int64_t rot_dims,
+                         at::Tensor positions, at::Tensor k_cache, at::Tensor v_cache,
+                         at::Tensor slots, double eps, bool v_unit_norm,
+                         const std::optional<at::Tensor>& v_inv_freq) {
+  HY_GPU(q);
+  const long T_ = q.size(0);
+  if (T_ == 0) return;
+  TORCH_CHECK(q.dim() == 3 && k.dim() == 3 && k.size(0) == T_ && k.size(2) == q.size(2));
+  HY_INNER(q); HY_INNER(k);
+  const int H = q.size(1), G = k.size(1), D = q.size(2);
+  TORCH_CHECK(q.stride(1) == D && k.stride(1) == D, "heads must be packed");
+  const auto dt = q.scalar_type();
+  TORCH_CHECK(k.scalar_type() == dt && k_cache.scalar_type() == dt && v_cache.scalar_type() == dt);
+  TORCH_CHECK(k_cache.dim() == 4 && k_cache.is_contiguous() && k_cache.size(1) == G &&
+              k_cache.size(3) == D, "key cache must be [blocks, G, block, D]");
+  const int bs = k_cache.size(2), DV = v_cache.size(3);
+  TORCH_CHECK(v_cache.dim() == 4 && v_cache.is_contiguous() && v_cache.size(0) == k_cache.size(0) &&
+              v_cache.size(1) == G && v_cache.size(2) == bs, "value cache must be [blocks, G, block, DV]");
+  const void* v_ptr = nullptr;
+  long v_stride = 0;
+  if (v_opt.has_value()) {
+    const at::Tensor& v = *v_opt;
+    HY_INNER(v);
+    TORCH_CHECK(v.dim() == 3 && v.size(0) == T_ && v.size(1) == G && v.size(2) == DV &&
+                v.stride(1) == DV && v.scalar_type() == dt, "v must be [T, G, DV], heads packed");
+    v_ptr = v.data_ptr();
+    v_stride = v.stride(0);
+  } else {
+    TORCH_CHECK(DV == D && !v_unit_norm && !v_inv_freq.has_value(),
+                "values that are the raw keys have the keys' size and pass unchanged");
+  }
+  auto weight_ptr = [&](const std::optional<at::Tensor>& w) -> const void* {
+    if (!w.has_value()) return nullptr;
+    TORCH_CHECK(w->is_cuda() && w->is_contiguous() && w->numel() == D && w->scalar_type() == dt,
+                "a head norm weight must be [D] in the activations' dtype");
+    return w->data_ptr();
+  };
+  const void* qw = weight_ptr(q_w);
+  const void* kw = weight_ptr(k_w);
+  auto table_ptr = [&](const std::optional<at::Tensor>& t, int dims) -> const float* {
+    TORCH_CHECK(t.has_value() && t->is_cuda() && t->scalar_type() == at::kFloat &&
+                t->is_contiguous() && t->numel() == dims / 2, "a rotary table must be fp32 [dims / 2]");
+    return t->data_ptr<float>();
+  };
+  TORCH_CHECK(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= D, "rot_dims must be even, at most D");
+  const float* table = rot_dims ? table_ptr(inv_freq, (int)rot_dims) : nullptr;
+  const float* v_table = nullptr;
+  if (v_inv_freq.has_value()) {
+    TORCH_CHECK(DV % 2 == 0, "rotated values need an even size");
+    v_table = table_ptr(v_inv_freq, DV);
+  }
+  TORCH_CHECK(rot_dims <= 2 * 64 * kRopePairs && D - rot_dims <= 64 * kRopeTail &&
+              DV <= 64 * kRopeTail && (!v_table || DV <= 2 * 64 * kRopePairs),
+              "head size beyond what a wave holds in registers");
+  TORCH_CHECK(positions.scalar_type() == at::kLong && positions.is_contiguous() &&
+              positions.numel() == T_ && positions.is_cuda());
+  TORCH_CHECK(slots.scalar_type() == at::kLong && slots.is_contiguous() && slots.numel() == T_ &&
+              slots.is_cuda());
+  const size_t lds = sizeof(float) * (size_t)(rot_dims + DV);
+  hy_dispatch(q, "qkv_norm_rope_cache", [&]<typename T>() {
+    hipLaunchKernelGGL(qkv_norm_rope_cache_kernel<T>, dim3(T_), dim3(256), lds, hy_stream(),
+                       reinterpret_cast<T*>(q.data_ptr()), q.stride(0),
+                       reinterpret_cast<const T*>(k.data_ptr()), k.stride(0),
+                       reinterpret_cast<const T*>(v_ptr), v_stride,
+                       reinterpret_cast<const T*>(qw), reinterpret_cast<const T*>(kw), table,
+                       (int)rot_dims, v_table, positions.data_ptr<long>(),
+                       reinterpret_cast<T*>(k_cache.data_ptr()),
+                       reinterpret_cast<T*>(v_cache.data_ptr()), slots.data_ptr<long>(), H, G, D, DV,
+                       bs, (float)eps, (int)v_unit_norm);
+  });
+}
+
+void rotate_heads(at::Tensor x, at::Tensor positions, at::Tensor inv_freq, bool inverse) {
+  HY_GPU(x);
+  const long T_ = x.size(0);
+  if (T_ == 0) return;
+  TORCH_CHECK(x.dim() == 3 && x.is_contiguous() && x.size(2) % 2 == 0, "x must be contiguous [T, H, n], n even");
+  const int H = x.size(1), n = x.size(2);
+  HY_F32(inv_freq);
+  TORCH_CHECK(inv_freq.numel() == n / 2);
+  TORCH_CHECK(positions.scalar_type() == at::kLong && positions.is_contiguous() &&
+              positions.numel() == T_ && positions.is_cuda());
+  hy_dispatch(x, "rotate_heads", [&]<typename T>() {
+    hipLaunchKernelGGL(rotate_heads_kernel<T>, dim3(T_), dim3(256), sizeof(float) * n, hy_stream(),
+                       reinterpret_cast<T*>(x.data_ptr()), positions.data_ptr<long>(),
+                       inv_freq.data_ptr<float>(), H, n, inverse ? -1.0f : 1.0f);
+  });
+}
+
+// out fp32 [3, T, H]; gates fp32 [T, 2H]; m_state fp32 [slots, H]
+void mlstm_gates(at::Tensor out, at::Tensor gates, double cap, at::Tensor m_state, at::Tensor cu,
+                 at::Tensor slots, at::Tensor fresh) {
+  HY_F32(gates);
+  const long T_ = gates.size(0);
+  if (T_ == 0) return;
+  TORCH_CHECK(gates.dim() == 2 && gates.size(1) % 2 == 0);
+  const int H = gates.size(1) / 2;
+  HY_F32(out);
+  TORCH_CHECK(out.dim() == 3 && out.size(0) == 3 && out.size(1) == T_ && out.size(2) == H);
+  const SeqDims d = seq_check(cu, slots, fresh, m_state);
+  TORCH_CHECK(m_state.dim() == 2 && m_state.size(1) == H && cap > 0.0, "m_state [slots, H] fp32");
+  hipLaunchKernelGGL(mlstm_gates_kernel, dim3(d.B, H), dim3(256), 0, hy_stream(),
+                     out.data_ptr<float>(), gates.data_ptr<float>(), (float)cap,
+                     m_state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(),
+                     fresh.data_ptr<int>(), H, T_);
+}
+
+// The recurrence kernel in its scalar-gate mode: q, k [T, H, D], v [T, H, DV]
+// (row-strided views, heads packed); decay, write fp32 [T, H]; o fp32
+// [T, H, DV + 1]; state fp32 [slots, H, D, DV + 1].
+void matrix_memory(at::Tensor o, at::Tensor q, at::Tensor k, at::Tensor v, at::Tensor decay,
+                   at::Tensor write, at::Tensor state, at::Tensor cu, at::Tensor slots,
+                   at::Tensor fresh, double q_scale) {
+  HY_GPU(q);
+  const long T_ = q.size(0);
+  if (T_ == 0) return;
+  TORCH_CHECK(q.dim() == 3 && k.sizes() == q.sizes() && v.dim() == 3);
+  HY_INNER(q); HY_INNER(k); HY_INNER(v);
+  const int H = q.size(1), D = q.size(2), DVin = v.size(2), DV = DVin + 1;
+  TORCH_CHECK(v.size(0) == T_ && v.size(1) == H);
+  TORCH_CHECK(q.stride(1) == D && k.stride(1) == D && v.stride(1) == DVin, "heads must be packed");
+  HY_F32(decay); HY_F32(write);
+  TORCH_CHECK(decay.dim() == 2 && decay.size(0) == T_ && decay.size(1) == H &&
+              write.sizes() == decay.sizes(), "decay and write must be fp32 [T, H]");
+  TORCH_CHECK(o.scalar_type() == at::kFloat && o.is_contiguous() && o.dim() == 3 &&
+              o.size(0) == T_ && o.size(1) == H && o.size(2) == DV);
+  const SeqDims sd = seq_check(cu, slots, fresh, state);
+  TORCH_CHECK(state.dim() == 4 && state.size(1) == H && state.size(2) == D && state.size(3) == DV,
+              "state [slots, H, D, DV + 1] fp32");
+  TORCH_CHECK(D <= 256, "key size above 256 is not supported");
+  const auto dt = q.scalar_type();
+  TORCH_CHECK(k.scalar_type() == dt && v.scalar_type() == dt);
+  const dim3 grid((DV + kGlaCols - 1) / kGlaCols, H, sd.B);
+  hy_dispatch(q, "matrix_memory", [&]<typename T>() {
+    auto launch = [&]<int DPL>() {
+      hipLaunchKernelGGL((gla_recurrence_kernel<T, DPL>), grid, dim3(256), 0, hy_stream(),
+                         o.data_ptr<float>(),
+                         reinterpret_cast<const T*>(q.data_ptr()), q.stride(0),
+                         reinterpret_cast<const T*>(k.data_ptr()), k.stride(0),
+                         reinterpret_cast<const T*>(v.data_ptr()), v.stride(0),
+                         static_cast<const T*>(nullptr), 0L, static_cast<const float*>(nullptr),
+                         state.data_ptr<float>(), cu.data_ptr<int>(), slots.data_ptr<int>(),
+                         fresh.data_ptr<int>(), H, D, DV, 1.0f, (float)q_scale,
+                         static_cast<const float*>(nullptr), 0, decay.data_ptr<float>(),
+                         write.data_ptr<float>(), 1);
+    };
+    if (D <= 32) launch.template operator()<2>();
+    else if (D <= 64) launch.template operator()<4>();
+    else if (D <= 128) launch.template operator()<8>();
+    else launch.template operator()<16>();
+  });
+}
+
+void mlstm_out_norm_gate(at::Tensor out, at::Tensor o, at::Tensor floor_, at::Tensor weight,
+                         at::Tensor gate, double eps) {
+  HY_GPU(o);
+  TORCH_CHECK(o.dim() == 3 && o.scalar_type() == at::kFloat && o.is_contiguous() && o.size(2) >= 2);
+  const long T_ = o.size(0);
+  if (T_ == 0) return;
+  const int H = o.size(1), DV = o.size(2) - 1;
+  HY_F32(floor_);
+  TORCH_CHECK(floor_.numel() == T_ * H);
+  TORCH_CHECK(out.dim() == 2 && out.is_contiguous() && out.size(0) == T_ && out.size(1) == (long)H * DV);
+  TORCH_CHECK(gate.dim() == 2 && gate.size(0) == T_ && gate.size(1) == (long)H * DV &&
+              gate.stride(1) == 1 && gate.scalar_type() == out.scalar_type());
+  TORCH_CHECK(weight.numel() == (long)H * DV && weight.is_contiguous() &&
+              weight.scalar_type() == out.scalar_type());
+  hy_dispatch(out, "mlstm_out_norm_gate", [&]<typename T>() {
+    hipLaunchKernelGGL(mlstm_out_norm_gate_kernel<T>, dim3(T_), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(out.data_ptr()), o.data_ptr<float>(),
+                       floor_.data_ptr<float>(), reinterpret_cast<const T*>(weight.data_ptr()),
+                       reinterpret_cast<const T*>(gate.data_ptr()), gate.stride(0), H, DV, (float)eps);
+  });
+}
+
+void dual_norm_mean(at::Tensor out, at::Tensor a, at::Tensor w_a, at::Tensor b, at::Tensor w_b,
+                    double eps) {
+  HY_GPU(a);
+  TORCH_CHECK(a.dim() == 2 && a.is_contiguous() && b.is_contiguous() && out.is_contiguous() &&
+              b.sizes() == a.sizes() && out.sizes() == a.sizes());
+  const long rows = a.size(0);
+  const int W = a.size(1);
+  if (rows == 0) return;
+  const auto dt = a.scalar_type();
+  TORCH_CHECK(b.scalar_type() == dt && out.scalar_type() == dt && w_a.scalar_type() == dt &&
+              w_b.scalar_type() == dt && w_a.is_contiguous() && w_b.is_contiguous() &&
+              w_a.numel() == W && w_b.numel() == W);
+  hy_dispatch(a, "dual_norm_mean", [&]<typename T>() {
+    hipLaunchKernelGGL(dual_norm_mean_kernel<T>, dim3(rows), dim3(256), 0, hy_stream(),
+                       reinterpret_cast<T*>(out.data_ptr()), reinterpret_cast<const T*>(a.data_ptr()),
+                       reinterpret_cast<const T*>(w_a.data_ptr()),
+                       reinterpret_cast<const T*>(b.data_ptr()),
+                       reinterpret_cast<const T*>(w_b.data_ptr()), W, (float)eps);
+  });
+}
+
+void unary_act(at::Tensor out, at::Tensor in, int64_t act) {
+  HY_GPU(in);
+  TORCH_CHECK(in.is_contiguous() && out.is_contiguous() && out.sizes() == in.sizes() &&
+              out.scalar_type() == in.scalar_type());
+  TORCH_CHECK(act == kActRelu2 || act == kActGeluErf, "unknown activation");
+  const long n = in.numel();
+  if (n == 0) return;
+  TORCH_CHECK(reinterpret_cast<uintptr_t>(in.data_ptr()) % 16 == 0 &&
+              reinterpret_cast<uintptr_t>(out.data_ptr()) % 16 == 0, "unary_act: 16-byte aligned tensors");
+  const int grid = (int)std::min<long>((n / 8 + 255) / 256 + 1, 8192);
+  hy_dispatch(in, "unary_act", [&]<typename T>() {
+    auto launch = [&]<int ACT>() {
+      hipLaunchKernelGGL((unary_act_kernel<T, ACT>), dim3(grid), dim3(256), 0, hy_stream(),
+                         reinterpret_cast<T*>(out.data_ptr()), reinterpret_cast<const T*>(in.data_ptr()), n);
+    };
+    if (act == kActRelu2) launch.template operator()<kActRelu2>();
+    else launch.template operator()<kActGeluErf>();
+  });
+}
+
 }  // namespace
 
+
 TORCH_LIBRARY(llmq_amd_hybrid, m) {
-  m.def("rmsnorm_cast(Tensor(a!) out, Tensor input, Tensor weight, float eps, float offset) -> ()");
-  m.def("sandwich_norm_res32(Tensor(a!) x, Tensor(b!) residual, Tensor w_post, Tensor w_pre, float eps, float offset) -> ()");
+  m.def("rmsnorm_cast(Tensor(a!) out, Tensor input, Tensor weight, float eps, float offset, int groups=1) -> ()");
+  m.def("sandwich_norm_res32(Tensor(a!) x, Tensor(b!) residual, Tensor w_post, Tensor w_pre, float eps, float offset, int groups=1) -> ()");
   m.def("act_and_mul(Tensor(a!) out, Tensor input, bool gelu) -> ()");
   m.def("qknorm_vmix_cache(Tensor(a!) q, Tensor k, Tensor v, Tensor q_w, Tensor k_w, Tensor? v_first, float lam, Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor slots, float eps) -> ()");
-  m.def("paged_attn_prefill(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor cu_q, Tensor q_start, int max_q, int span, float scale, int mask_mode, int pos_stride, int bias_mode) -> ()");
-  m.def("paged_attn_decode(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor context_lens, int span, float scale, int mask_mode, int bias_mode) -> ()");
+  m.def("paged_attn_prefill(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor cu_q, Tensor q_start, int max_q, int span, float scale, int mask_mode, int pos_stride, int bias_mode, int keep_first=0, Tensor? sink=None, float softcap=0.0) -> ()");
+  m.def("paged_attn_decode(Tensor(a!) out, Tensor q, Tensor? gate, Tensor k_cache, Tensor? v_cache, Tensor? bias, Tensor block_tables, Tensor context_lens, int span, float scale, int mask_mode, int bias_mode, int keep_first=0, Tensor? sink=None, float softcap=0.0) -> ()");
   m.def("gla_recurrence(Tensor(a!) o, Tensor q, Tensor? k, Tensor v, Tensor z, Tensor z_bias, Tensor(b!) state, Tensor cu, Tensor slots, Tensor fresh, float tau, Tensor? lower, bool q_silu, float q_scale) -> ()");
   m.def("gla_out_norm_gate(Tensor(a!) out, Tensor o, Tensor weight, Tensor? gate, float eps) -> ()");
   m.def("latent_rope_pack(Tensor(a!) out, Tensor q, Tensor q_lat, Tensor ckr, Tensor c_w, Tensor inv_freq, Tensor positions, Tensor(b!) k_cache, Tensor slots, int dim, int rot_dims, bool interleaved, float eps) -> ()");
@@ -1078,10 +1346,17 @@ TORCH_LIBRARY(llmq_amd_hybrid, m) {
   m.def("depth_mix_norm(Tensor(a!) out, Tensor(b!) stack, int n, Tensor coef, Tensor y, Tensor? y2, float a1, float a2, Tensor weight, float eps) -> ()");
   m.def("kv_scatter(Tensor k, Tensor v, Tensor(a!) k_cache, Tensor(b!) v_cache, Tensor slots) -> ()");
   m.def("mingru_scan(Tensor(a!) out, Tensor z, Tensor u, Tensor g, Tensor z_b, Tensor u_b, Tensor(b!) state, Tensor cu, Tensor slots, Tensor fresh) -> ()");
-  m.def("causal_conv_silu(Tensor(a!) out, Tensor x, Tensor weight, Tensor bias, Tensor(b!) tail, Tensor cu, Tensor slots, Tensor fresh) -> ()");
+  m.def("causal_conv_silu(Tensor(a!) out, Tensor x, Tensor weight, Tensor? bias, Tensor(b!) tail, Tensor cu, Tensor slots, Tensor fresh, bool silu=True) -> ()");
   m.def("selective_scan(Tensor(a!) out, Tensor x, Tensor dt, Tensor dt_b, Tensor A, Tensor Bm, Tensor Cm, Tensor D, Tensor z, Tensor(b!) state, Tensor cu, Tensor slots, Tensor fresh) -> ()");
-  m.def("softmax_topk(Tensor(a!) idx, Tensor(b!) w, Tensor logits, int top, float scale) -> ()");
+  m.def("softmax_topk(Tensor(a!) idx, Tensor(b!) w, Tensor logits, int top, float scale, Tensor? correction=None, bool renorm=False) -> ()");
   m.def("clamp_swish_mul(Tensor(a!) out, Tensor input, float limit) -> ()");
+  m.def("qkv_norm_rope_cache(Tensor(a!) q, Tensor k, Tensor? v, Tensor? q_w, Tensor? k_w, Tensor? inv_freq, int rot_dims, Tensor positions, Tensor(b!) k_cache, Tensor(c!) v_cache, Tensor slots, float eps, bool v_unit_norm, Tensor? v_inv_freq) -> ()");
+  m.def("rotate_heads(Tensor(a!) x, Tensor positions, Tensor inv_freq, bool inverse) -> ()");
+  m.def("mlstm_gates(Tensor(a!) out, Tensor gates, float cap, Tensor(b!) m_state, Tensor cu, Tensor slots, Tensor fresh) -> ()");
+  m.def("matrix_memory(Tensor(a!) o, Tensor q, Tensor k, Tensor v, Tensor decay, Tensor write, Tensor(b!) state, Tensor cu, Tensor slots, Tensor fresh, float q_scale) -> ()");
+  m.def("mlstm_out_norm_gate(Tensor(a!) out, Tensor o, Tensor floor, Tensor weight, Tensor gate, float eps) -> ()");
+  m.def("dual_norm_mean(Tensor(a!) out, Tensor a, Tensor w_a, Tensor b, Tensor w_b, float eps) -> ()");
+  m.def("unary_act(Tensor(a!) out, Tensor input, int act) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(llmq_amd_hybrid, CUDA, m) {
@@ -1111,4 +1386,11 @@ TORCH_LIBRARY_IMPL(llmq_amd_hybrid, CUDA, m) {
   m.impl("selective_scan", &selective_scan);
   m.impl("softmax_topk", &softmax_topk);
   m.impl("clamp_swish_mul", &clamp_swish_mul);
+  m.impl("qkv_norm_rope_cache", &qkv_norm_rope_cache);
+  m.impl("rotate_heads", &rotate_heads);
+  m.impl("mlstm_gates", &mlstm_gates);
+  m.impl("matrix_memory", &matrix_memory);
+  m.impl("mlstm_out_norm_gate", &mlstm_out_norm_gate);
+  m.impl("dual_norm_mean", &dual_norm_mean);
+  m.impl("unary_act", &unary_act);
 }

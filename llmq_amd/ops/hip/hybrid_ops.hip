@@ -6,4 +6,5 @@
 #include "seqmix.hip"
 #include "latent_moe.hip"
 #include "scan_mix.hip"
+#include "memory_mix.hip"
 #include "hybrid_bindings.cpp"

@@ -365,7 +365,8 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
     T* __restrict__ out, const T* __restrict__ x, long x_stride, const float* __restrict__ w,
     const float* __restrict__ bias, const float* __restrict__ tail,
     const int* __restrict__ cu, const int* __restrict__ slots, const int* __restrict__ fresh,
-    int B, int C, int K, int rows_per_thread) {
+    int B, int C, int K, int rows_per_thread, int silu) {
+  // bias may be null; silu == 0 leaves the convolution's result as it is
   const int c = blockIdx.x * 256 + threadIdx.x;
   if (c >= C) return;
   const int total = cu[B];
@@ -375,7 +376,7 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
   float wk[kConvMaxTaps], win[kConvMaxTaps];
 #pragma unroll
   for (int k = 0; k < kConvMaxTaps; ++k) wk[k] = k < K ? w[(long)c * K + k] : 0.f;
-  const float bc = bias[c];
+  const float bc = bias ? bias[c] : 0.f;
   int b = 0;
   while (cu[b + 1] <= r0) ++b;   // the sequence of row r0 (empty sequences skipped)
   bool load_window = true;
@@ -416,7 +417,7 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(
 #pragma unroll
         for (int k = 0; k < kConvMaxTaps; ++k)
           if (k == K - 1) acc += wk[k] * xv;
-        out[(long)r * C + c] = from_f32<T>(acc * sigmoid_f(acc));
+        out[(long)r * C + c] = from_f32<T>(silu ? acc * sigmoid_f(acc) : acc);
 #pragma unroll
         for (int k = 0; k < kConvMaxTaps - 2; ++k)
           if (k < K - 2) win[k] = win[k + 1];
@@ -640,7 +641,10 @@ __global__ __launch_bounds__(64 * NC) void selective_scan_kernel(
 // 64 * 32 experts).
 __global__ __launch_bounds__(256) void softmax_topk_kernel(
     int* __restrict__ idx_out, float* __restrict__ w_out, const float* __restrict__ logits,
-    long rows, int E, int top, float scale) {
+    long rows, int E, int top, float scale, const float* __restrict__ correction, int renorm) {
+  // correction [E] (or null): the choice is made on s + correction, the
+  // weights stay the plain scores. renorm: the chosen scores are divided by
+  // their sum (+ 1e-20) before the scale.
   const int lane = threadIdx.x & 63;
   const long tok = blockIdx.x * 4L + (threadIdx.x >> 6);
   if (tok >= rows) return;
@@ -664,6 +668,7 @@ __global__ __launch_bounds__(256) void softmax_topk_kernel(
     for (int e = lane, n = 0; e < E; e += 64, ++n) {
       if (taken & (1u << n)) continue;
       float v = z[e];
+      if (correction) v = expf(v - mx) / sum + correction[e];
       if (!(v == v)) v = -3.0e38f;   // a NaN logit still yields a valid index
       if (v > best || best_e == 0x7fffffff) {   // ascending e: the first of equals stays
         best = v;
@@ -682,8 +687,16 @@ __global__ __launch_bounds__(256) void softmax_topk_kernel(
     if ((best_e & 63) == lane) taken |= 1u << (best_e >> 6);
     if (lane == 0) {
       idx_out[tok * top + k] = best_e;
-      w_out[tok * top + k] = expf(best - mx) / sum * scale;
+      w_out[tok * top + k] = expf((correction ? z[best_e] : best) - mx) / sum;
     }
+  }
+  if (lane == 0) {
+    float total = 1.0f;
+    if (renorm) {
+      total = 1e-20f;
+      for (int k = 0; k < top; ++k) total += w_out[tok * top + k];
+    }
+    for (int k = 0; k < top; ++k) w_out[tok * top + k] = w_out[tok * top + k] / total * scale;
   }
 }
 

@@ -15,14 +15,19 @@
 // Residual stream in fp32, sublayer I/O in T.
 
 // out = rmsnorm(in) * (w + offset); TI/TO may differ (fp32 stream -> T).
+// A row normed in `groups` equal consecutive parts is `groups` rows of
+// `hidden` elements each to these kernels; part g reads the weights from
+// g * hidden on.
 template <typename TI, typename TO>
 __global__ void rmsnorm_cast_kernel(TO* __restrict__ out, const TI* __restrict__ in,
                                     long in_stride, const TO* __restrict__ weight, int hidden,
-                                    float eps, float offset) {
+                                    float eps, float offset, int groups) {
   __shared__ float red[4];
   const long row = blockIdx.x;
-  const TI* x = in + row * in_stride;
+  const int part = (int)(row % groups);
+  const TI* x = in + (row / groups) * in_stride + (long)part * hidden;
   TO* o = out + row * hidden;
+  weight += (long)part * hidden;
   float ss = 0.f;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     const float f = to_f32(x[i]);
@@ -42,9 +47,11 @@ template <typename T>
 __global__ void sandwich_norm_res32_kernel(T* __restrict__ x, float* __restrict__ residual,
                                            const T* __restrict__ w_post,
                                            const T* __restrict__ w_pre, int hidden,
-                                           float eps, float offset) {
+                                           float eps, float offset, int groups) {
   __shared__ float red[4];
   const long row = blockIdx.x;
+  w_post += (row % groups) * hidden;
+  w_pre += (row % groups) * hidden;
   T* xr = x + row * hidden;
   float* rr = residual + row * hidden;
   float ss = 0.f;
@@ -74,9 +81,11 @@ template <int CH>
 __global__ __launch_bounds__(256) void sandwich_norm_res32_vec_kernel(
     __hip_bfloat16* __restrict__ x, float* __restrict__ residual,
     const __hip_bfloat16* __restrict__ w_post, const __hip_bfloat16* __restrict__ w_pre,
-    int hidden, float eps, float offset) {
+    int hidden, float eps, float offset, int groups) {
   __shared__ float red[4];
   const long row = blockIdx.x;
+  w_post += (row % groups) * hidden;
+  w_pre += (row % groups) * hidden;
   __hip_bfloat16* xr = x + row * hidden;
   float* rr = residual + row * hidden;
   float xv[CH][8], rv[CH][8];
@@ -256,6 +265,28 @@ DEVINL float dist_bias(const float* __restrict__ bias, int bias_len, int mode, i
   return bias[(long)h * bias_len + min(d, bias_len - 1)];
 }
 
+// Score cap: c * tanh(s / c). FAST (bf16 models): through the hardware
+// exponential, 1 - 2 / (e^(2x) + 1); fp32 models: tanhf.
+template <bool FAST>
+DEVINL float cap_score(float s, float cap) {
+  const float x = s / cap;
+  return cap * (FAST ? 1.0f - 2.0f / (__expf(2.0f * x) + 1.0f) : tanhf(x));
+}
+
+// Kept first tokens (window mask only): besides its window a query sees every
+// key j < keep_first. The keys below min(keep_first, first key of the window
+// of the tile's first query) are walked as tiles of their own before the
+// window's tiles, cut at that bound so no key is visited twice.
+//
+// Softmax sink: after the last key a head's denominator gains exp(sink[h]),
+// a term without a key or a value.
+DEVINL void add_sink(float& m, float& l, float& rescale, float sink) {
+  const float m_new = fmaxf(m, sink);
+  rescale = m > -INFINITY ? expf(m - m_new) : 0.f;
+  l = l * rescale + expf(sink - m_new);
+  m = m_new;
+}
+
 template <typename T, int NV>
 __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     T* __restrict__ out, long out_stride,
@@ -267,7 +298,8 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     const int* __restrict__ cu_q,          // [B+1]
     const int* __restrict__ q_start,       // [B] position of a sequence's first query
     int H, int G, int D, int DV, int block_size, int span, float scale,
-    int v_row, int mask_mode, int bias_mode) {
+    int v_row, int mask_mode, int bias_mode, int keep_first, const float* __restrict__ sink,
+    float softcap) {
   extern __shared__ float smem[];
   const int b = blockIdx.z, h = blockIdx.y;
   const int row0 = cu_q[b];
@@ -305,8 +337,11 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
   }
   const int* bt = block_tables + (long)b * bt_stride;
   const int lo = mask_first_key(pos0, span, mask_mode);
-  for (int kt = lo; kt <= pos_last; kt += kAttnKT) {
-    const int nk = min(kAttnKT, pos_last + 1 - kt);
+  const int first_end = min(keep_first, lo);   // keys [0, first_end): kept, before every window
+  for (int kt = first_end > 0 ? 0 : lo; kt <= pos_last;) {
+    const bool in_first = kt < first_end;
+    const int kt_next = (in_first && kt + kAttnKT >= first_end) ? lo : kt + kAttnKT;
+    const int nk = min(kAttnKT, (in_first ? first_end : pos_last + 1) - kt);
     __syncthreads();
     for (int idx = tid; idx < nk * D; idx += 256) {
       const int jj = idx / D, d = idx % D;
@@ -341,9 +376,10 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
     for (int r = 0; r < 4; ++r) {
       const int i = pos0 + w * 4 + r;
       const bool vis = lane < nk && (w * 4 + r) < rows && key <= i &&
-                       key >= mask_first_key(i, span, mask_mode);
+                       (key >= mask_first_key(i, span, mask_mode) || key < keep_first);
+      const float sr = softcap > 0.f ? cap_score<sizeof(T) == 2>(s[r], softcap) : s[r];
       const float sc = !vis ? -INFINITY
-          : bias ? s[r] + dist_bias<sizeof(T) == 2>(bias, bias_len, bias_mode, h, i - key) : s[r];
+          : bias ? sr + dist_bias<sizeof(T) == 2>(bias, bias_len, bias_mode, h, i - key) : sr;
       const float tmax = wave_reduce_max(sc);
       const float m_new = fmaxf(m[r], tmax);
       float p = 0.f, corr = 1.f;
@@ -378,12 +414,19 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
         acc[3][n] += a3;
       }
     }
+    kt = kt_next;
   }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     const int rr = w * 4 + r;
     if (rr >= rows) continue;
     const long trow = row0 + r0 + rr;
+    if (sink) {
+      float rescale;
+      add_sink(m[r], l[r], rescale, sink[h]);
+#pragma unroll
+      for (int n = 0; n < NV; ++n) acc[r][n] *= rescale;
+    }
     float gs = 1.f;
     if (gate) gs = 1.0f / (1.0f + expf(-to_f32(gate[trow * g_stride + h])));
     const float inv = gs / l[r];
@@ -424,7 +467,8 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ cu_q, const int* __restrict__ q_start,
     int H, int G, int D, int DV, int block_size, int span, float scale,
-    int v_row, int mask_mode, int ps, int n_split, float* __restrict__ part, int bias_mode) {
+    int v_row, int mask_mode, int ps, int n_split, float* __restrict__ part, int bias_mode,
+    int keep_first, const float* __restrict__ sink, float softcap) {
   // n_split > 1: the grid's y dimension carries (key split, head); a
   // workgroup walks only its share of the key tiles and writes its
   // unnormalised output, running maximum and sum to `part`
@@ -532,8 +576,14 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     kt0 += sp * chunk * kMfmaKT;
     key_end = min(pos_last, kt0 + chunk * kMfmaKT - 1);
   }
+  // kept first tokens (never together with key splits): their tiles come first
+  const int win0 = kt0;
+  const int first_end = min(keep_first, win0);
+  if (first_end > 0) kt0 = 0;
   if (kt0 <= key_end) fetch(kt0);
-  for (int kt = kt0; kt <= key_end; kt += kMfmaKT) {
+  for (int kt = kt0; kt <= key_end;) {
+    const bool in_first = kt < first_end;
+    const int kt_next = (in_first && kt + kMfmaKT >= first_end) ? win0 : kt + kMfmaKT;
     __syncthreads();
 #pragma unroll
     for (int i = 0; i < KS; ++i) {
@@ -557,8 +607,9 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
           : d < bias_len ? bias_h[d] : 0.f;
     }
     __syncthreads();
-    if (kt + kMfmaKT <= key_end) fetch(kt + kMfmaKT);
-    const bool active = wave_rows && kt <= wave_last && kt + kMfmaKT - 1 >= wave_lo;
+    if (kt_next <= key_end) fetch(kt_next);
+    const bool active = wave_rows && kt <= wave_last &&
+                        (in_first || kt + kMfmaKT - 1 >= wave_lo);
     if (active) {
       sm_f32x4 s[4];
 #pragma unroll
@@ -580,8 +631,11 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
 #pragma unroll
         for (int ct = 0; ct < 4; ++ct) {
           const int key = kt + ct * 16 + col;
-          const bool vis = key >= lorow[reg] && key <= irow[reg];
-          sv[ct] = vis ? s[ct][reg] * scale + brow[-ct * 16] : -INFINITY;
+          const bool vis = key <= irow[reg] &&
+              (in_first ? key < first_end : (key >= lorow[reg] || key < keep_first));
+          float sc = s[ct][reg] * scale;
+          if (softcap > 0.f) sc = cap_score<true>(sc, softcap);
+          sv[ct] = vis ? sc + brow[-ct * 16] : -INFINITY;
           tmax = fmaxf(tmax, sv[ct]);
         }
         tmax = fmaxf(tmax, __shfl_xor(tmax, 1, WAVE));
@@ -632,6 +686,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
         }
       }
     }
+    kt = kt_next;
   }
 #pragma unroll
   for (int reg = 0; reg < 4; ++reg) {
@@ -643,6 +698,12 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
     const int r = w * 16 + kgrp * 4 + reg;
     if (r >= rows) continue;
     const long trow = row0 + r0 + r;
+    if (sink && n_split == 1) {
+      float rescale;
+      add_sink(m[reg], ll, rescale, sink[h]);
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) o[dt][reg] *= rescale;
+    }
     if (n_split > 1) {
       float* pr = part + ((trow * H + h) * n_split + sp) * (long)(DV + 2);
 #pragma unroll
@@ -720,7 +781,8 @@ __global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
     const int* __restrict__ block_tables, int bt_stride,
     const int* __restrict__ context_lens,
     int H, int G, int D, int DV, int block_size, int span, float scale,
-    int v_row, int mask_mode, int bias_mode) {
+    int v_row, int mask_mode, int bias_mode, int keep_first, const float* __restrict__ sink,
+    float softcap) {
   extern __shared__ __align__(16) float smem[];
   const int h0 = blockIdx.x * HPW, b = blockIdx.y;
   const int g = h0 / (H / G);
@@ -748,8 +810,14 @@ __global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
 #pragma unroll
     for (int n = 0; n < NV; ++n) acc[hh][n] = 0.f;
   }
-  for (int kt = lo + w * 64; kt <= i; kt += NW * 64) {
-    const int nk = min(64, i + 1 - kt);
+  // tiles: first the kept keys below the window, then the window's
+  const int first_end = min(keep_first, lo);
+  const int n_first = (first_end + 63) / 64;
+  const int n_tiles = n_first + (i - lo) / 64 + 1;
+  for (int tile = w; tile < n_tiles; tile += NW) {
+    const bool in_first = tile < n_first;
+    const int kt = in_first ? tile * 64 : lo + (tile - n_first) * 64;
+    const int nk = min(64, (in_first ? first_end : i + 1) - kt);
     const int key = kt + lane;
     long base = 0;
     float sc[HPW];
@@ -784,9 +852,11 @@ __global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
         }
       }
 #pragma unroll
-      for (int hh = 0; hh < HPW; ++hh)
-        sc[hh] = bias ? s[hh] + dist_bias<sizeof(T) == 2>(bias, bias_len, bias_mode, h0 + hh, i - key)
-                      : s[hh];
+      for (int hh = 0; hh < HPW; ++hh) {
+        const float sr = softcap > 0.f ? cap_score<sizeof(T) == 2>(s[hh], softcap) : s[hh];
+        sc[hh] = bias ? sr + dist_bias<sizeof(T) == 2>(bias, bias_len, bias_mode, h0 + hh, i - key)
+                      : sr;
+      }
     }
     float p[HPW];
 #pragma unroll
@@ -835,6 +905,10 @@ __global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
 #pragma unroll
     for (int ww = 0; ww < NW; ++ww) mm = fmaxf(mm, Ms[ww * HPW + hh]);
     float a = 0.f, ll = 0.f;
+    if (sink) {
+      mm = fmaxf(mm, sink[h0 + hh]);
+      ll = expf(sink[h0 + hh] - mm);
+    }
 #pragma unroll
     for (int ww = 0; ww < NW; ++ww) {
       const float mw = Ms[ww * HPW + hh];
@@ -856,6 +930,12 @@ __global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
 //     w = k;
 //   HGRN2 (lower != null): a = l + (1 - l) * sigmoid(z + z_bias), w = 1 - a
 //     (no key is read).
+//   matrix memory (hdecay != null): per token and head ONE decay and one
+//     write strength, computed beforehand (fp32 [T, H]): a = hdecay[t, h] on
+//     every key channel, w = hwrite[t, h] * k; z is not read. With ones_col the
+//     value gets one more column that is always 1, so the state's last column
+//     accumulates the written keys alone (an mLSTM's normaliser vector) and
+//     the output's last column is its product with q.
 // q enters as q_scale * q, or q_scale * silu(q) with q_silu.
 //
 // Value columns evolve independently, so the grid splits DV: a workgroup owns
@@ -886,8 +966,12 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
     const int* __restrict__ fresh,          // [B]
     int H, int D, int DV, float inv_tau, float q_scale,
     const float* __restrict__ lower,        // [H*D] or null
-    int q_silu) {
+    int q_silu,
+    const float* __restrict__ hdecay,       // [T, H] or null
+    const float* __restrict__ hwrite,       // [T, H] (with hdecay)
+    int ones_col) {                         // v has DV - 1 columns; column DV - 1 is 1
   constexpr int DP = 16 * DPL;          // padded key channels
+  const int DVin = DV - (ones_col ? 1 : 0);
   __shared__ __align__(16) float qs[kGlaTB * DP];
   __shared__ __align__(16) float ks[kGlaTB * DP];
   __shared__ __align__(16) float as[kGlaTB * DP];
@@ -927,15 +1011,21 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
         const long row = row0 + t0 + tt;
         rq[j] = to_f32(q[row * q_stride + (long)h * D + d]);
         if (k) rk[j] = to_f32(k[row * k_stride + (long)h * D + d]);
-        rz[j] = to_f32(z[row * z_stride + (long)h * D + d]);
+        if (hdecay) {
+          rz[j] = hdecay[row * H + h];
+          rk[j] *= hwrite[row * H + h];
+        } else {
+          rz[j] = to_f32(z[row * z_stride + (long)h * D + d]);
+        }
       }
     }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const int idx = tid + 256 * j;
       const int tt = idx / kGlaCols, gc = blockIdx.x * kGlaCols + idx % kGlaCols;
-      rv[j] = (tt < nt && gc < DV)
-          ? to_f32(v[(long)(row0 + t0 + tt) * v_stride + (long)h * DV + gc]) : 0.f;
+      rv[j] = (tt < nt && gc < DVin)
+          ? to_f32(v[(long)(row0 + t0 + tt) * v_stride + (long)h * DVin + gc])
+          : (tt < nt && gc < DV) ? 1.f : 0.f;
     }
   };
   if (n > 0) fetch(0);
@@ -951,7 +1041,9 @@ __global__ __launch_bounds__(256) void gla_recurrence_kernel(
         if constexpr (std::is_same_v<T, float>) qv = qv / (1.0f + expf(-qv));
         else qv = qv / (1.0f + __expf(-qv));
       }
-      if (d < D && lower) {
+      if (hdecay) {
+        av = rz[j];                     // 0 on padded rows and channels
+      } else if (d < D && lower) {
         const float zz = rz[j] + z_bias[h * D + d];
         const float lo = lower[h * D + d];
         float sg;

@@ -45,14 +45,15 @@ def rotate_half(x, first_pos, base, dims, sign=1.0):
     n = x.shape[0]
     half = dims // 2
     out = x.clone()
-    for i in range(half):
-        f = base ** (-2.0 * i / dims)
-        for r in range(n):
-            a = sign * (first_pos + r) * f
-            c, s = math.cos(a), math.sin(a)
-            u, v = x[r, ..., i].clone(), x[r, ..., i + half].clone()
-            out[r, ..., i] = u * c - v * s
-            out[r, ..., i + half] = v * c + u * s
+    if not half:
+        return out
+    freq = torch.tensor([base ** (-2.0 * i / dims) for i in range(half)], dtype=F64)
+    pos = torch.arange(first_pos, first_pos + n, dtype=F64)
+    ang = sign * pos.view(n, *([1] * (x.dim() - 1))) * freq
+    c, s = torch.cos(ang), torch.sin(ang)
+    u, v = x[..., :half], x[..., half:dims]
+    out[..., :half] = u * c - v * s
+    out[..., half:dims] = v * c + u * s
     return out
 
 
@@ -222,3 +223,13 @@ def forward(cfg, t, ids, layer_outputs=None):
             layer_outputs.append(x.clone())
     x = group_norm(x, t["final.norm"], eps, groups)
     return x @ t["embed"].T
+
+
+def greedy(cfg, t, ids, n):
+    """n greedy continuations of ids, each from a whole forward pass."""
+    ids, out = list(ids), []
+    for _ in range(n):
+        nxt = int(forward(cfg, t, ids)[-1].argmax())
+        out.append(nxt)
+        ids.append(nxt)
+    return out

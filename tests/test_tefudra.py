@@ -1,0 +1,848 @@
+"""Tefudra (windowed attention beside a matrix memory) against the plain
+oracle in tefudra_oracle.py.
+
+Every test builds its own small configuration and random checkpoint, loads
+it through the engine's own entry points (config reader, weight loader,
+scheduler, cache and state managers) and compares logits with the oracle.
+The scenarios run on the CPU (torch reference ops) and, marked ``gpu``, on
+the HIP kernels in fp32 (sharp) and bf16.
+
+Expert routing is a discrete choice: a bf16 run rounds the router's input,
+so a near-tie may fall the other way than in the float64 oracle. Whole-model
+bf16 scenarios therefore use mixtures in which every expert is chosen (the
+scores still weigh the outputs); the choice itself is checked in fp32 at
+model level and at op level, where the oracle sees the same inputs.
+"""
+
+from __future__ import annotations
+
+import json
+import math
+
+import pytest
+import torch
+
+import tefudra_oracle as oracle
+from llmq_amd import ops
+from llmq_amd.engine.config import EngineConfig
+from llmq_amd.engine.engine import LLMEngine
+from llmq_amd.engine.sampling_params import SamplingParams
+
+
+# --------------------------------------------------------------- fixtures --
+
+def moe_cfg(experts=5, identity=2, top=3, ff=24, shared=20):
+    cfg = {"kind": "moe", "expert": {"ff": ff},
+           "router": {"experts": experts, "identity": identity, "top": top}}
+    if shared:
+        cfg["shared"] = {"ff": shared}
+    return cfg
+
+
+def dense(ff=40):
+    return {"kind": "dense", "ff": ff}
+
+
+def attn(heads=4, kv_heads=2, dim=16, rot_dims=8, base=10000.0, size=12, keep=3, scale=0.3,
+         mlp="dense", **extra):
+    mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": scale,
+             "rot": {"base": base, "dims": rot_dims}, "mask": {"size": size, "keep_first": keep}}
+    return dict({"type": "attention", "mixer": mixer, "mlp": dense() if mlp == "dense" else mlp},
+                **extra)
+
+
+def par(heads=4, kv_heads=2, dim=8, vdim=12, rot_dims=8, base=5000.0, size=10, scale=0.35,
+        softcap=5.0, conv=3, mheads=2, mdim=8, mvdim=12, gate_cap=8.0, mlp="dense", **extra):
+    left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale,
+            "rot": {"base": base, "dims": rot_dims}, "mask": {"size": size}, "softcap": softcap,
+            "conv": conv}
+    right = {"heads": mheads, "dim": mdim, "vdim": mvdim, "gate_cap": gate_cap}
+    return dict({"type": "parallel", "mixer": {"left": left, "right": right},
+                 "mlp": dense() if mlp == "dense" else mlp}, **extra)
+
+
+def make_config(layers, width=48, vocab=128, eps=1e-5, groups=3):
+    return {"architecture": "Tefudra", "layers": layers, "norm": {"eps": eps, "groups": groups},
+            "vocab": vocab, "width": width}
+
+
+def make_tensors(cfg, seed=0):
+    g = torch.Generator().manual_seed(seed)
+
+    def rnd(*shape, std=1.0, mean=0.0):
+        return (torch.randn(shape, generator=g) * std + mean).to(torch.bfloat16)
+
+    def lin(out, inn, gain=1.0):
+        return rnd(out, inn, std=gain / math.sqrt(inn))
+
+    W, V = cfg["width"], cfg["vocab"]
+    t = {"embed": rnd(V, W), "final.norm": rnd(W, std=0.1, mean=0.9)}
+    for i, layer in enumerate(cfg["layers"]):
+        if "weights_of" in layer:
+            continue
+        p, m = f"l{i}.", layer["mixer"]
+        t[p + "norm1"] = rnd(W, std=0.1, mean=1.1)
+        t[p + "norm1b"] = rnd(W, std=0.1, mean=0.6)
+        if layer["type"] == "attention":
+            H, G, D = m["heads"], m["kv_heads"], m["dim"]
+            t[p + "mix.q"], t[p + "mix.k"] = lin(H * D, W, 2.0), lin(G * D, W, 2.0)
+            t[p + "mix.q.norm"] = rnd(D, std=0.2, mean=1.5)
+            t[p + "mix.k.norm"] = rnd(D, std=0.2, mean=1.5)
+            t[p + "mix.sink"] = rnd(H, std=1.0, mean=1.0)
+            t[p + "mix.o"] = lin(W, H * D, 2.0)
+        else:
+            a, r = m["left"], m["right"]
+            H, G, D, DV, K = a["heads"], a["kv_heads"], a["dim"], a["vdim"], a["conv"]
+            for name, rows in (("q", H * D), ("k", G * D), ("v", G * DV)):
+                t[f"{p}mix.left.{name}"] = lin(rows, W, 2.5)
+                t[f"{p}mix.left.{name}.b"] = rnd(rows, std=0.3)
+                t[f"{p}mix.left.{name}.conv"] = rnd(rows, K, std=0.9 / math.sqrt(K))
+            t[p + "mix.left.o"], t[p + "mix.left.o.b"] = lin(W, H * DV, 2.0), rnd(W, std=0.3)
+            MH, MD, MV = r["heads"], r["dim"], r["vdim"]
+            t[p + "mix.right.q"], t[p + "mix.right.k"] = lin(MH * MD, W, 2.0), lin(MH * MD, W, 2.0)
+            t[p + "mix.right.v"], t[p + "mix.right.g"] = lin(MH * MV, W, 2.0), lin(MH * MV, W, 2.0)
+            t[p + "mix.right.o"] = lin(W, MH * MV, 2.0)
+            t[p + "mix.right.norm"] = rnd(MH * MV, std=0.1, mean=1.0)
+            t[p + "mix.right.i"], t[p + "mix.right.i.b"] = lin(MH, W, 3.0), rnd(MH, std=1.0)
+            t[p + "mix.right.f"] = lin(MH, W, 3.0)
+            t[p + "mix.right.f.b"] = rnd(MH, std=1.0, mean=2.0)
+            t[p + "mix.left.out"] = rnd(W, std=0.1, mean=1.0)
+            t[p + "mix.right.out"] = rnd(W, std=0.1, mean=0.8)
+        mlp = layer["mlp"]
+        if mlp is None:
+            continue
+        t[p + "norm2"] = rnd(W, std=0.1, mean=1.0)
+        t[p + "norm2b"] = rnd(W, std=0.1, mean=0.6)
+        if mlp["kind"] == "dense":
+            t[p + "mlp.up"], t[p + "mlp.down"] = lin(mlp["ff"], W, 2.0), lin(W, mlp["ff"], 1.5)
+        else:
+            r, ff = mlp["router"], mlp["expert"]["ff"]
+            n = r["experts"] + r.get("identity", 0)
+            t[p + "mlp.router"] = lin(n, W, 2.0)
+            t[p + "mlp.correction"] = rnd(n, std=0.15)
+            for e in range(r["experts"]):
+                t[f"{p}mlp.e{e}.up"], t[f"{p}mlp.e{e}.down"] = lin(ff, W, 2.0), lin(W, ff, 2.0)
+            if mlp.get("shared"):
+                sf = mlp["shared"]["ff"]
+                t[p + "mlp.shared.up"], t[p + "mlp.shared.down"] = lin(sf, W, 2.0), lin(W, sf, 1.5)
+    return t
+
+
+def write_checkpoint(path, cfg, tensors):
+    from safetensors.torch import save_file
+
+    path.mkdir(parents=True, exist_ok=True)
+    (path / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in tensors.items()}, str(path / "model.safetensors"))
+    return str(path)
+
+
+def mixed_layers(route):
+    """Every switch at once: both mixers, both feed-forwards, a layer without
+    one, grouped and ungrouped heads, q/k size != v size, full and partial
+    rotation, windows of different sizes, and a layer on another's weights."""
+    moe = (lambda **kw: moe_cfg(experts=5, identity=2, top=3, **kw)) if route else \
+        (lambda **kw: moe_cfg(experts=3, identity=1, top=4, **kw))
+    return [
+        par(mlp="dense"),
+        attn(mlp=moe()),
+        par(heads=3, kv_heads=3, dim=16, vdim=8, rot_dims=6, size=25, softcap=2.0, conv=4,
+            mheads=3, mdim=4, mvdim=20, mlp=None),
+        par(heads=2, kv_heads=1, dim=12, vdim=12, rot_dims=12, size=7, conv=2, mheads=1, mdim=16,
+            mvdim=8, mlp=moe(shared=None)),
+        attn(heads=2, kv_heads=2, dim=24, rot_dims=24, size=20, keep=0, scale=0.2, mlp="dense"),
+        attn(mlp=moe(), weights_of=1),
+    ]
+
+
+def tokens_for(n, vocab, seed):
+    g = torch.Generator().manual_seed(3000 + seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+DEVICES = [
+    pytest.param(("cpu", "float32"), id="cpu"),
+    pytest.param(("cuda", "float32"), id="hip-fp32", marks=pytest.mark.gpu),
+    pytest.param(("cuda", "bfloat16"), id="hip-bf16", marks=pytest.mark.gpu),
+]
+
+
+def make_engine(path, target, blocks=64, block_size=16, max_seqs=4, prefill_budget=4096,
+                max_len=1024):
+    device, dtype = target
+    return LLMEngine(EngineConfig(
+        model=path, device=device, dtype=dtype, max_num_seqs=max_seqs, max_model_len=max_len,
+        num_kv_blocks=blocks, kv_block_size=block_size, max_prefill_tokens=prefill_budget))
+
+
+def tolerance(target):
+    """(worst row, mean over rows) of the relative rms error. fp32 is the
+    sharp comparison; bf16 rounds every GEMM input and output of a deep
+    stack and only has to stay at rounding level."""
+    return (8e-2, 2.5e-2) if target[1] == "bfloat16" else (2e-4, 5e-5)
+
+
+def assert_close(got, want, target, what=""):
+    got, want = got.double().cpu(), want.double()
+    err = (got - want).pow(2).mean(-1).sqrt() / want.pow(2).mean(-1).sqrt()
+    worst, mean = float(err.max()), float(err.mean())
+    lim_worst, lim_mean = tolerance(target)
+    assert worst < lim_worst, f"{what}: worst row error {worst:.3e} at row {int(err.argmax())}"
+    assert mean < lim_mean, f"{what}: mean row error {mean:.3e}"
+
+
+def replay(engine, rid, toks, cuts, end=True):
+    """One request alone, cut into the given portion sizes; all logits."""
+    out, at = [], 0
+    for n in cuts:
+        last = at + n == len(toks)
+        out.append(engine.replay_step(
+            [{"id": rid, "tokens": toks[at:at + n], "want": list(range(n))}],
+            end=[rid] if (last and end) else []))
+        at += n
+    assert at == len(toks)
+    return torch.cat(out)
+
+
+def f64(tensors):
+    return {k: v.double() for k, v in tensors.items()}
+
+
+_MODELS = {}
+
+
+@pytest.fixture(scope="module")
+def mixed_model(tmp_path_factory):
+    """(config, tensors, path) of the all-switches model; bf16 targets get the
+    variant in which every expert is chosen."""
+    def get(target):
+        route = target[1] != "bfloat16"
+        if route not in _MODELS:
+            cfg = make_config(mixed_layers(route))
+            tensors = make_tensors(cfg, seed=11)
+            path = write_checkpoint(tmp_path_factory.mktemp("tf") / "m", cfg, tensors)
+            _MODELS[route] = (cfg, f64(tensors), path)
+        return _MODELS[route]
+    return get
+
+
+_WANT = {}
+
+
+def oracle_logits(cfg, tensors, toks):
+    key = (id(tensors), tuple(toks))
+    if key not in _WANT:
+        _WANT[key] = oracle.forward(cfg, tensors, toks)
+    return _WANT[key]
+
+
+def dev_dtype(target):
+    return target[0], (torch.bfloat16 if target[1] == "bfloat16" else torch.float32)
+
+
+# ------------------------------------------------------ config and layout --
+
+def test_config_reader_takes_everything_from_config(tmp_path):
+    from llmq_amd.engine.model_specs import resolve_spec
+
+    cfg = make_config(mixed_layers(True))
+    tensors = make_tensors(cfg)
+    path = write_checkpoint(tmp_path / "m", cfg, tensors)
+    spec = resolve_spec(path)
+    assert spec.family == "tefudra" and spec.num_layers == 6 and spec.hidden_size == 48
+    assert (spec.rms_eps, spec.norm_groups) == (1e-5, 3)
+    assert [ls.mixer.kind for ls in spec.layers] == [
+        "parallel", "sink_attention", "parallel", "parallel", "sink_attention", "sink_attention"]
+    a = spec.layers[1].mixer
+    assert (a.heads, a.kv_heads, a.dim, a.scale, a.window, a.keep_first) == (4, 2, 16, 0.3, 12, 3)
+    assert (a.rot.base, a.rot.dims) == (10000.0, 8)
+    assert spec.layers[4].mixer.keep_first == 0 and spec.layers[4].mixer.rot.dims == 24
+    lt, rt = spec.layers[2].mixer.left, spec.layers[2].mixer.right
+    assert (lt.heads, lt.kv_heads, lt.dim, lt.vdim, lt.window, lt.softcap, lt.conv) == \
+        (3, 3, 16, 8, 25, 2.0, 4)
+    assert (lt.rot.base, lt.rot.dims) == (5000.0, 6)
+    assert (rt.heads, rt.dim, rt.vdim, rt.gate_cap) == (3, 4, 20, 8.0)
+    e = spec.layers[1].moe
+    assert (e.experts, e.identity, e.top, e.ff, e.shared_ff) == (5, 2, 3, 24, 20)
+    assert spec.layers[2].ff == 0 and spec.layers[2].moe is None
+    assert spec.layers[3].moe.shared_ff == 0 and spec.layers[0].ff == 40
+    assert spec.layers[5].weights_of == 1 and spec.owner(5) == 1
+    assert spec.param_count() == sum(v.numel() for v in tensors.values())
+    # every layer owns key/value pages, a shared-weights layer too; parallel
+    # layers own the memory, its running maximum and the convolution's tail
+    eng = make_engine(path, ("cpu", "float32"))
+    assert eng.model.layers[5] is eng.model.layers[1]
+    assert eng.kv_cache.k[5] is not eng.kv_cache.k[1]
+    assert eng.kv_cache.k[1].shape[1:] == (2, 16, 16) and eng.kv_cache.v[1].shape[1:] == (2, 16, 16)
+    assert eng.kv_cache.k[2].shape[1:] == (3, 16, 16) and eng.kv_cache.v[2].shape[1:] == (3, 16, 8)
+    assert eng.state_cache.state[1] is None
+    mem, mx, tail = eng.state_cache.state[2]
+    assert mem.shape[1:] == (3, 4, 21) and mx.shape[1:] == (3,) and tail.shape[1:] == (3, 120)
+    with pytest.raises(ValueError):
+        resolve_spec(write_checkpoint(tmp_path / "bad", make_config([dict(attn(), type="lstm")]), {}))
+    with pytest.raises(ValueError):
+        resolve_spec(write_checkpoint(tmp_path / "bad2", make_config([attn(weights_of=3)]), {}))
+
+
+# ------------------------------------------------------ mechanisms alone --
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("layers,kw", [
+    ([attn(mlp=None)], {}),
+    ([attn(keep=0, size=9, mlp=None)], {"groups": 1}),
+    ([attn(heads=3, kv_heads=3, dim=8, rot_dims=8, size=64, keep=2, mlp=None)], {}),  # window > prompt
+    ([attn(heads=6, kv_heads=1, dim=20, rot_dims=4, size=5, keep=7, mlp=None)], {}),  # keep > window
+    ([par(mlp=None)], {}),
+    ([par(softcap=30.0, conv=1, rot_dims=4, mlp=None)], {"groups": 1}),
+    ([par(heads=1, kv_heads=1, dim=32, vdim=32, rot_dims=32, size=1, mheads=1, mdim=32, mvdim=32,
+          mlp=None)], {}),
+    ([par(heads=6, kv_heads=2, dim=4, vdim=20, rot_dims=2, conv=8, mheads=4, mdim=12, mvdim=4,
+          gate_cap=2.0, mlp=None)], {"groups": 6}),
+    ([attn(mlp=dense(56))], {}),
+    ([attn(mlp=moe_cfg(experts=4, identity=2, top=6))], {}),
+    ([attn(mlp=moe_cfg(experts=3, identity=0, top=3, shared=None))], {}),
+    ([attn(mlp=moe_cfg(experts=1, identity=1, top=2))], {}),
+    ([par(mlp=None), par(mlp=None, weights_of=0), attn(mlp=None), attn(mlp=None, weights_of=2)], {}),
+], ids=["sink", "sink-plain-window", "sink-wide-window", "sink-keep-beyond-window", "pair",
+        "pair-loose-cap-no-conv", "pair-ones", "pair-wide", "dense", "moe-all", "moe-no-identity",
+        "moe-single", "shared-weights"])
+def test_mechanism_alone(tmp_path, target, layers, kw):
+    cfg = make_config(layers, **kw)
+    tensors = make_tensors(cfg, seed=3)
+    path = write_checkpoint(tmp_path / "m", cfg, tensors)
+    toks = tokens_for(37, cfg["vocab"], 1)
+    eng = make_engine(path, target)
+    eng.model.taps = []
+    got = replay(eng, "a", toks, [37])
+    taps = []
+    want = oracle.forward(cfg, f64(tensors), toks, taps)
+    for i, (g, w) in enumerate(zip(eng.model.taps, taps)):
+        assert_close(g, w, target, f"stream after layer {i}")
+    assert_close(got, want, target, "logits")
+
+
+@pytest.mark.parametrize("target", DEVICES)
+def test_sizes_that_fit_no_vector_width(tmp_path, target):
+    layers = [par(heads=3, kv_heads=1, dim=6, vdim=10, rot_dims=2, size=9, conv=3, mheads=3, mdim=5,
+                  mvdim=7, mlp=moe_cfg(experts=3, identity=1, top=4, ff=9, shared=7)),
+              attn(heads=3, kv_heads=1, dim=10, rot_dims=6, size=11, keep=2, mlp=dense(13))]
+    cfg = make_config(layers, width=27, vocab=61, groups=3)
+    tensors = make_tensors(cfg, seed=5)
+    path = write_checkpoint(tmp_path / "m", cfg, tensors)
+    toks = tokens_for(41, 61, 2)
+    want = oracle.forward(cfg, f64(tensors), toks)
+    eng = make_engine(path, target)
+    assert_close(replay(eng, "a", toks, [41]), want, target, "whole")
+    assert_close(replay(eng, "b", toks, [7, 1, 1, 30, 2]), want, target, "portions")
+
+
+@pytest.mark.parametrize("target", DEVICES[:2])
+@pytest.mark.parametrize("experts,identity,top", [(5, 2, 1), (5, 2, 2), (7, 3, 3), (2, 0, 1),
+                                                  (13, 4, 4), (3, 5, 2)])
+def test_expert_choice_in_the_model(tmp_path, target, experts, identity, top):
+    cfg = make_config([attn(mlp=moe_cfg(experts=experts, identity=identity, top=top)),
+                       par(mlp=moe_cfg(experts=experts, identity=identity, top=top, shared=None))])
+    tensors = make_tensors(cfg, seed=experts * 10 + top)
+    path = write_checkpoint(tmp_path / "m", cfg, tensors)
+    toks = tokens_for(33, cfg["vocab"], 6)
+    assert_close(replay(make_engine(path, target), "a", toks, [30, 1, 1, 1]),
+                 oracle.forward(cfg, f64(tensors), toks), target,
+                 f"{experts}+{identity} experts, top {top}")
+
+
+# ------------------------------------------- schedules: cuts, batches, reuse --
+
+@pytest.mark.parametrize("target", DEVICES)
+def test_prefill_equals_token_by_token(mixed_model, target):
+    cfg, tensors, path = mixed_model(target)
+    toks = tokens_for(90, cfg["vocab"], 2)
+    want = oracle_logits(cfg, tensors, toks)
+    eng = make_engine(path, target)
+    assert_close(replay(eng, "w", toks, [90]), want, target, "whole prompt")
+    assert_close(replay(eng, "d", toks, [1] * 90), want, target, "token by token")
+    assert eng.allocator.num_free == eng.allocator.num_blocks
+    assert eng.slot_allocator.num_free == 4
+
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("cuts", [
+    [2] * 45,
+    [1, 2, 3, 5, 8, 13, 21, 34, 3],
+    [16, 16, 16, 16, 16, 10],                  # at page borders
+    [15, 2, 15, 17, 31, 1, 1, 8],              # around page borders
+    [64, 1, 1, 1, 1, 1, 1, 1, 1, 1, 17],
+    [3, 87],
+], ids=["twos", "growing", "pages", "around-pages", "decode-then-portion", "short-first"])
+def test_portions(mixed_model, target, cuts):
+    cfg, tensors, path = mixed_model(target)
+    toks = tokens_for(90, cfg["vocab"], 3)
+    want = oracle_logits(cfg, tensors, toks)
+    eng = make_engine(path, target)
+    assert_close(replay(eng, "c", toks, cuts), want, target, f"cuts {cuts}")
+
+
+@pytest.mark.parametrize("target", DEVICES)
+def test_mixed_batches_equal_alone_and_reuse(mixed_model, target):
+    """Six unequal requests through four slots and a pool that cannot hold
+    them all at once: portions beside single tokens, requests that pause,
+    blocks and slots handed on to later requests."""
+    cfg, tensors, path = mixed_model(target)
+    lens = {"a": 70, "b": 9, "c": 41, "d": 130, "e": 25, "f": 3}
+    toks = {r: tokens_for(n, cfg["vocab"], 10 + i) for i, (r, n) in enumerate(lens.items())}
+    want = {r: oracle_logits(cfg, tensors, t) for r, t in toks.items()}
+    eng = make_engine(path, target, blocks=14, block_size=16)
+    at = {r: 0 for r in lens}
+    got = {r: [] for r in lens}
+    plan = [
+        {"a": 33, "b": 2, "c": 17},
+        {"a": 1, "b": 1, "c": 24, "d": 40},
+        {"a": 1, "b": 6, "d": 2},              # c pauses at its end; b ends
+        {"a": 35, "d": 1, "e": 25},            # e takes b's slot and blocks
+        {"d": 1, "e": 0, "c": 0},
+        {"d": 86, "f": 3},                     # a, c, e ended; f reuses
+    ]
+    ends = [[], [], ["b"], ["a", "e"], ["c"], ["d", "f"]]
+    slots_seen = set()
+    for step, end in zip(plan, ends):
+        entries = []
+        for r, n in step.items():
+            if n:
+                entries.append({"id": r, "tokens": toks[r][at[r]:at[r] + n], "want": list(range(n))})
+        out = eng.replay_step(entries, end=[])
+        for s in eng._seqs.values():
+            slots_seen.add(s.state_slot)
+        eng.replay_step([], end=end)
+        k = 0
+        for ent in entries:
+            n = len(ent["tokens"])
+            got[ent["id"]].append(out[k:k + n])
+            at[ent["id"]] += n
+            k += n
+    assert at == lens
+    assert slots_seen <= {0, 1, 2, 3}
+    for r in lens:
+        assert_close(torch.cat(got[r]), want[r], target, f"request {r}")
+    assert eng.allocator.num_free == 14 and eng.slot_allocator.num_free == 4
+
+
+@pytest.mark.parametrize("target", DEVICES)
+def test_stale_pages_and_slots_do_not_leak(mixed_model, target):
+    """A request that runs in blocks and a slot another one just left sees
+    nothing of it: same logits as in a fresh engine."""
+    cfg, tensors, path = mixed_model(target)
+    first = tokens_for(64, cfg["vocab"], 30)
+    second = tokens_for(50, cfg["vocab"], 31)
+    want = oracle_logits(cfg, tensors, second)
+    eng = make_engine(path, target, blocks=4, max_seqs=1)
+    replay(eng, "x", first, [60, 1, 1, 1, 1])
+    assert_close(replay(eng, "y", second, [3, 1, 1, 45]), want, target, "after reuse")
+
+
+@pytest.mark.parametrize("target", DEVICES)
+def test_long_decode_across_pages_and_windows(mixed_model, target):
+    cfg, tensors, path = mixed_model(target)
+    toks = tokens_for(5 + 150, cfg["vocab"], 4)
+    want = oracle_logits(cfg, tensors, toks)
+    eng = make_engine(path, target)
+    assert_close(replay(eng, "l", toks, [5] + [1] * 150), want, target, "long decode")
+
+
+@pytest.mark.parametrize("target", DEVICES)
+def test_first_tokens(mixed_model, target):
+    """One-token and two-token requests, and the tokens before any window,
+    convolution or kept range is full."""
+    cfg, tensors, path = mixed_model(target)
+    eng = make_engine(path, target)
+    for n in (1, 2, 3, 4):
+        toks = tokens_for(n, cfg["vocab"], 70 + n)
+        assert_close(replay(eng, f"n{n}", toks, [n]), oracle_logits(cfg, tensors, toks), target,
+                     f"{n} tokens")
+
+
+# ------------------------------------------ edges made visible by design --
+
+def _needle(device, dtype, key_pos, query_pos, decode, window, keep, sink=None, softcap=0.0,
+            H=2, G=1, D=16, DV=8, block_size=16, raw=8.0):
+    """Every key scores 0 and has value 0, but the needle at key_pos: raw score
+    `raw`, value 1 in channel 1. The output's channel 1 is then the softmax
+    weight the needle gets. Pages are handed out in reverse order."""
+    n = query_pos + 1
+    nblocks = (n + block_size - 1) // block_size
+    kc = torch.zeros(nblocks + 2, G, block_size, D, dtype=dtype)
+    vc = torch.zeros(nblocks + 2, G, block_size, DV, dtype=dtype)
+    table = torch.arange(nblocks + 1, 0, -1, dtype=torch.int32).view(1, -1)   # reversed pages
+    b, o = int(table[0, key_pos // block_size]), key_pos % block_size
+    kc[b, :, o, 0] = raw
+    vc[b, :, o, 1] = 1.0
+    kc, vc, table = kc.to(device), vc.to(device), table.to(device)
+    sk = None if sink is None else torch.full((H,), sink, dtype=torch.float32, device=device)
+    kw = dict(keep_first=keep, sink=sk, softcap=softcap)
+    if decode:
+        q = torch.zeros(1, H, D, dtype=dtype, device=device)
+        q[0, :, 0] = 1.0
+        out = ops.window_attn_decode(
+            q, kc, vc, DV, table, torch.tensor([n], dtype=torch.int32, device=device), window, 1.0,
+            **kw)
+        return float(out[0, H - 1, 1])
+    start = max(0, query_pos - 4)            # a portion whose last row is the query
+    rows = query_pos - start + 1
+    q = torch.zeros(rows, H, D, dtype=dtype, device=device)
+    q[:, :, 0] = 1.0
+    out = ops.window_attn_prefill(
+        q, kc, vc, DV, table, torch.tensor([0, rows], dtype=torch.int32, device=device),
+        torch.tensor([start], dtype=torch.int32, device=device), rows, window, 1.0, **kw)
+    return float(out[-1, H - 1, 1])
+
+
+def _needle_weight(key_pos, query_pos, window, keep, sink=None, softcap=0.0, raw=8.0):
+    """Dense formula: the needle's softmax weight among the keys the query sees."""
+    seen = [j for j in range(query_pos + 1) if query_pos - j < window or j < keep]
+    if key_pos not in seen:
+        return 0.0
+    s = raw if not softcap else softcap * math.tanh(raw / softcap)
+    den = math.exp(s) + (len(seen) - 1) + (math.exp(sink) if sink is not None else 0.0)
+    return math.exp(s) / den
+
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("decode", [False, True], ids=["portion", "single"])
+def test_window_edges_kept_tokens_and_far_keys(target, decode):
+    """The needle just inside and just outside the window, just inside and
+    just outside the kept first tokens, at page borders and at tile borders
+    of the kernels, among hundreds of keys."""
+    device, dtype = dev_dtype(target)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+    window, keep = 300, 5
+    for query_pos in (299, 300, 700, 1023):
+        lo = query_pos - window + 1
+        keys = {0, keep - 1, keep, keep + 1, 15, 16, 63, 64, lo - 1, lo, lo + 1, query_pos - 64,
+                query_pos - 1, query_pos}
+        for key_pos in sorted(k for k in keys if 0 <= k <= query_pos):
+            got = _needle(device, dtype, key_pos, query_pos, decode, window, keep, sink=2.0)
+            want = _needle_weight(key_pos, query_pos, window, keep, sink=2.0)
+            assert abs(got - want) < tol * max(want, 0.05), (query_pos, key_pos, got, want)
+    # a window without kept tokens, a kept range longer than a tile, no sink
+    for window, keep, query_pos in ((40, 0, 500), (33, 70, 400), (64, 64, 129)):
+        lo = query_pos - window + 1
+        for key_pos in (0, keep - 1, keep, lo - 1, lo, query_pos):
+            if key_pos < 0:
+                continue
+            got = _needle(device, dtype, key_pos, query_pos, decode, window, keep)
+            want = _needle_weight(key_pos, query_pos, window, keep)
+            assert abs(got - want) < tol * max(want, 0.05), (window, keep, query_pos, key_pos)
+
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("decode", [False, True], ids=["portion", "single"])
+def test_sink_and_score_cap(target, decode):
+    """A sink far above and far below the scores, and a cap that flattens the
+    needle's score."""
+    device, dtype = dev_dtype(target)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+    for sink in (-30.0, 0.0, 7.5, 40.0):
+        got = _needle(device, dtype, 90, 100, decode, 50, 2, sink=sink)
+        want = _needle_weight(90, 100, 50, 2, sink=sink)
+        assert abs(got - want) < tol * max(want, 1e-3), (sink, got, want)
+    for cap in (1.0, 3.0, 50.0):
+        got = _needle(device, dtype, 90, 100, decode, 50, 0, softcap=cap)
+        want = _needle_weight(90, 100, 50, 0, softcap=cap)
+        assert abs(got - want) < tol * max(want, 1e-3), (cap, got, want)
+
+
+@pytest.mark.parametrize("target", DEVICES)
+def test_sink_is_per_head(target):
+    device, dtype = dev_dtype(target)
+    H, D = 3, 8
+    kc = torch.zeros(2, 1, 16, D, dtype=dtype, device=device)
+    vc = torch.ones(2, 1, 16, D, dtype=dtype, device=device)
+    q = torch.zeros(1, H, D, dtype=dtype, device=device)
+    sink = torch.tensor([-50.0, 0.0, math.log(9.0)], device=device)
+    table = torch.tensor([[1, 0]], dtype=torch.int32, device=device)
+    out = ops.window_attn_decode(q, kc, vc, D, table,
+                                 torch.tensor([9], dtype=torch.int32, device=device), 0, 1.0, sink=sink)
+    want = torch.tensor([1.0, 0.9, 0.5])
+    assert (out[0, :, 0].float().cpu() - want).abs().max() < 1e-2
+
+
+@pytest.mark.parametrize("target", DEVICES)
+def test_values_rotate_by_their_position_and_back(target):
+    """qkv_norm_rope_cache + rotate_heads: a value cached at position j and
+    read alone at position i comes out turned by j - i."""
+    device, dtype = dev_dtype(target)
+    G, D, DV, bs = 1, 8, 12, 16
+    from llmq_amd.engine.models.kosalorn import rotary_inv_freq
+
+    table_v = rotary_inv_freq(100.0, DV).to(device)
+    table_k = rotary_inv_freq(100.0, 4).to(device)
+    g = torch.Generator().manual_seed(5)
+    T = 40
+    q = torch.randn(T, 2, D, generator=g).to(dtype).to(device)
+    k = torch.randn(T, G, D, generator=g).to(dtype).to(device)
+    v = torch.randn(T, G, DV, generator=g).to(dtype).to(device)
+    kc = torch.zeros(4, G, bs, D, dtype=dtype, device=device)
+    vc = torch.zeros(4, G, bs, DV, dtype=dtype, device=device)
+    pos = torch.arange(T, dtype=torch.long, device=device)
+    slots = pos.clone()
+    slots[7] = -1                                     # a padding row writes nothing
+    q0 = q.clone()
+    ops.qkv_norm_rope_cache(q, k, v, None, None, table_k, 4, pos, kc, vc, slots, 1e-6,
+                            v_unit_norm=True, v_inv_freq=table_v)
+    cached = vc.permute(0, 2, 1, 3).reshape(-1, G, DV)[:T]
+    assert float(cached[7].abs().max()) == 0.0
+    back = ops.rotate_heads(cached.clone().contiguous(), pos, table_v, inverse=True)
+    unit = v.double() / (v.double().pow(2).mean(-1, keepdim=True) + 1e-6).sqrt()
+    keep = [i for i in range(T) if i != 7]
+    tol = 3e-2 if dtype == torch.bfloat16 else 1e-5
+    assert (back.double()[keep] - unit[keep]).abs().max().item() < tol
+    # q: unrotated channels pass, rotated pairs keep their length
+    assert (q[..., 4:] - q0[..., 4:]).abs().max().item() == 0.0
+    n0 = q0.double()[..., :4].pow(2).sum(-1)
+    assert ((q.double()[..., :4].pow(2).sum(-1) - n0).abs() / n0).max().item() < 10 * tol
+
+
+# ------------------------------------------------------ ops against oracle --
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("H,D,DV,lens", [(2, 8, 12, [70, 1, 3, 40]), (1, 32, 32, [300]),
+                                         (3, 5, 7, [17, 33]), (4, 64, 48, [5, 1, 1]),
+                                         (2, 16, 31, [1, 1, 1])])
+def test_matrix_memory_ops_against_token_by_token(target, H, D, DV, lens):
+    """mlstm_gates + matrix_memory + mlstm_out_norm_gate over unequal packed
+    sequences, each cut in two calls through its state slot, against the
+    plain recurrence over the whole sequence."""
+    device, dtype = dev_dtype(target)
+    g = torch.Generator().manual_seed(H * 100 + D)
+    B, cap, eps = len(lens), 6.0, 1e-5
+    full = [n * 2 + 1 for n in lens]
+    data = []
+    for n in full:
+        data.append(dict(
+            q=torch.randn(n, H, D, generator=g), k=torch.randn(n, H, D, generator=g),
+            v=torch.randn(n, H, DV, generator=g), gate=torch.randn(n, H * DV, generator=g),
+            gi=torch.randn(n, H, generator=g) * 3, gf=torch.randn(n, H, generator=g) * 3 + 2))
+    w = (torch.randn(H * DV, generator=g) * 0.1 + 1).to(dtype)
+    S = torch.full((B + 1, H, D, DV + 1), 7.0, device=device)       # stale contents
+    M = torch.full((B + 1, H), -3.0, device=device)
+    slots = torch.tensor(list(range(B - 1, -1, -1)), dtype=torch.int32, device=device)
+    outs = [[] for _ in range(B)]
+    for part in range(2):
+        spans = [(0, n) if part == 0 else (n, f) for n, f in zip(lens, full)]
+        cu = torch.tensor([0] + list(torch.tensor([e - s for s, e in spans]).cumsum(0)),
+                          dtype=torch.int32, device=device)
+        cat = lambda key, dt: torch.cat([d[key][s:e] for d, (s, e) in zip(data, spans)]).to(dt).to(device)
+        gates = torch.cat([cat("gi", torch.float32), cat("gf", torch.float32)], dim=1)
+        fresh = torch.full((B,), 1 - part, dtype=torch.int32, device=device)
+        decay, write, floor = ops.mlstm_gates(gates, cap, M, cu, slots, fresh)
+        o = ops.matrix_memory(cat("q", dtype), cat("k", dtype), cat("v", dtype), decay, write, S,
+                              cu, slots, fresh, D ** -0.5)
+        y = ops.mlstm_out_norm_gate(o, floor, w.to(device), cat("gate", dtype), eps, dtype)
+        for b in range(B):
+            outs[b].append(y[int(cu[b]):int(cu[b + 1])].cpu())
+    tol = 4e-2 if dtype == torch.bfloat16 else 2e-4
+    for b, d in enumerate(data):
+        r = {k: t.to(dtype).double() for k, t in d.items() if k not in ("gi", "gf")}
+        n = full[b]
+        gi = cap * torch.tanh(d["gi"].double() / cap)
+        gf = oracle.log_sigmoid(cap * torch.tanh(d["gf"].double() / cap))
+        want = torch.zeros(n, H, DV, dtype=torch.float64)
+        for a in range(H):
+            Sm, nv, mx = torch.zeros(D, DV, dtype=torch.float64), torch.zeros(D, dtype=torch.float64), 0.0
+            for t in range(n):
+                new = max(float(gf[t, a]) + mx, float(gi[t, a]))
+                df, di = math.exp(float(gf[t, a]) + mx - new), math.exp(float(gi[t, a]) - new)
+                Sm = df * Sm + di * torch.outer(r["k"][t, a], r["v"][t, a])
+                nv = df * nv + di * r["k"][t, a]
+                mx = new
+                qq = r["q"][t, a] * D ** -0.5
+                want[t, a] = (Sm.T @ qq) / (max(abs(float(nv @ qq)), math.exp(-mx)) + 1e-6)
+        want = oracle.rms(want, eps).reshape(n, H * DV) * w.double() * oracle.sigmoid(r["gate"])
+        got = torch.cat(outs[b]).double()
+        err = (got - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()
+        assert err < tol, (b, float(err))
+
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("E,top,T", [(7, 3, 9), (20, 4, 130), (2, 1, 5), (5, 5, 33)])
+def test_router_with_correction(target, E, top, T):
+    device, _ = dev_dtype(target)
+    g = torch.Generator().manual_seed(E + top)
+    logits = torch.randn(T, E, generator=g) * 2
+    corr = torch.randn(E, generator=g) * 0.3
+    idx, w = ops.softmax_topk(logits.to(device), top, 1.0, correction=corr.to(device), renorm=True)
+    s = torch.softmax(logits.double(), -1)
+    for t in range(T):
+        order = sorted(range(E), key=lambda e: (-(float(s[t, e]) + float(corr[e])), e))[:top]
+        assert idx[t].tolist() == order
+        want = s[t, order] / (s[t, order].sum() + 1e-20)
+        assert (w[t].double().cpu() - want).abs().max() < 1e-5
+
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("W,F,E,ident,top,T", [(48, 24, 5, 2, 3, 9), (40, 20, 3, 0, 2, 3),
+                                               (36, 10, 3, 3, 3, 130), (64, 32, 8, 2, 2, 700)])
+def test_expert_mixture_with_identity_experts(target, W, F, E, ident, top, T):
+    """Ungated GELU experts and identity experts through every form of the
+    expert op (sorted, and the batched form decode graphs use)."""
+    device, dtype = dev_dtype(target)
+    g = torch.Generator().manual_seed(W + T)
+    h = torch.randn(T, W, generator=g).to(dtype)
+    up = (torch.randn(E, F, W, generator=g) / math.sqrt(W)).to(dtype)
+    down = (torch.randn(E, W, F, generator=g) / math.sqrt(F)).to(dtype)
+    idx = torch.stack([torch.randperm(E + ident, generator=g)[:top] for _ in range(T)]).int()
+    w = torch.rand(T, top, generator=g) + 0.1
+    w = w / w.sum(-1, keepdim=True)
+    want = torch.zeros(T, W, dtype=torch.float64)
+    for t in range(T):
+        for j in range(top):
+            e = int(idx[t, j])
+            x = h[t].double()
+            y = oracle.gelu_erf(up[e].double() @ x) if e < E else None
+            want[t] += float(w[t, j]) * (down[e].double() @ y if e < E else x)
+    tol = 4e-2 if dtype == torch.bfloat16 else 2e-4
+    for sync_free in (False, True):
+        got = ops.moe_experts(h.to(device), idx.to(device), w.to(device), up.to(device),
+                              down.to(device), sync_free=sync_free, act="gelu_erf",
+                              weight_output=True, identity=ident)
+        err = (got.double().cpu() - want).pow(2).mean().sqrt() / want.pow(2).mean().sqrt()
+        assert err < tol, (sync_free, float(err))
+
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("W,groups", [(48, 3), (27, 3), (2048, 4), (2056, 1), (192, 4)])
+def test_grouped_norms_joins_and_activations(target, W, groups):
+    device, dtype = dev_dtype(target)
+    g = torch.Generator().manual_seed(W)
+    T, eps = 19, 1e-5
+    x = torch.randn(T, W, generator=g).to(dtype)
+    y = torch.randn(T, W, generator=g).to(dtype)
+    res = torch.randn(T, W, generator=g)
+    w1 = (torch.randn(W, generator=g) * 0.1 + 1).to(dtype)
+    w2 = (torch.randn(W, generator=g) * 0.1 + 0.7).to(dtype)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+
+    def close(got, want):
+        return (got.double().cpu() - want).abs().max().item() < tol * want.abs().max().item()
+
+    want_n = oracle.group_norm(res.double(), w1.double(), eps, groups)
+    assert close(ops.rmsnorm_cast(res.to(device), w1.to(device), eps, 0.0, dtype, groups), want_n)
+    r = res.clone().to(device)
+    h = ops.sandwich_norm_res32(x.clone().to(device), r, w1.to(device), w2.to(device), eps, 0.0, groups)
+    want_r = res.double() + oracle.group_norm(x.double(), w1.double(), eps, groups)
+    assert close(r, want_r)
+    assert close(h, oracle.group_norm(want_r, w2.double(), eps, groups))
+    want_m = 0.5 * (oracle.rms(x.double(), eps) * w1.double() + oracle.rms(y.double(), eps) * w2.double())
+    assert close(ops.dual_norm_mean(x.to(device), w1.to(device), y.to(device), w2.to(device), eps), want_m)
+    assert close(ops.unary_act(x.to(device), "relu2"), torch.clamp(x.double(), min=0) ** 2)
+    assert close(ops.unary_act(x.to(device), "gelu_erf"), oracle.gelu_erf(x.double()))
+
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("C,K", [(5, 4), (64, 3), (300, 8), (7, 2)])
+def test_plain_convolution_across_short_cuts(target, C, K):
+    """The convolution without bias and activation, its tail carried through
+    cuts shorter than its reach."""
+    device, dtype = dev_dtype(target)
+    g = torch.Generator().manual_seed(C * K)
+    n = 23
+    x = torch.randn(n, C, generator=g).to(dtype)
+    w = torch.randn(C, K, generator=g)
+    want = oracle.causal_conv(x.double(), w.double())
+    tail = torch.full((2, K - 1, C), 9.0, device=device)
+    got, at = [], 0
+    for cut in (1, 1, 2, 1, 5, 1, 12):
+        cu = torch.tensor([0, cut], dtype=torch.int32, device=device)
+        got.append(ops.causal_conv_silu(
+            x[at:at + cut].to(device), w.to(device), None, tail, cu,
+            torch.tensor([1], dtype=torch.int32, device=device),
+            torch.tensor([int(at == 0)], dtype=torch.int32, device=device), silu=False))
+        at += cut
+    tol = 3e-2 if dtype == torch.bfloat16 else 1e-5
+    assert (torch.cat(got).double().cpu() - want).abs().max().item() < tol * want.abs().max().item()
+
+
+# -------------------------------------------- generation and entry points --
+
+@pytest.mark.parametrize("target", DEVICES[:2])
+def test_greedy_generation_through_the_scheduler(mixed_model, target):
+    """add_request / step: the scheduler's own admission, chunked prefill
+    (a budget smaller than the prompts), decode batching and sampler."""
+    cfg, tensors, path = mixed_model(target)
+    prompts = {"p": tokens_for(21, cfg["vocab"], 40), "q": tokens_for(5, cfg["vocab"], 41),
+               "r": tokens_for(34, cfg["vocab"], 42)}
+    eng = make_engine(path, target, prefill_budget=16)
+    params = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    for rid, toks in prompts.items():
+        eng.add_request(rid, prompt_token_ids=toks, params=params)
+    got = {rid: [] for rid in prompts}
+    while eng.has_unfinished():
+        for out in eng.step():
+            got[out.request_id].extend(out.new_token_ids)
+    for rid, toks in prompts.items():
+        assert got[rid] == oracle.greedy(cfg, tensors, toks, 6), rid
+    assert eng.allocator.num_free == eng.allocator.num_blocks
+
+
+def test_preset_runs_through_generate():
+    eng = LLMEngine(EngineConfig(model="tiny-tefudra", device="cpu", max_num_seqs=2,
+                                 max_model_len=64, num_kv_blocks=8))
+    out = eng.generate_batch(["ab", "c"], SamplingParams(temperature=0.0, max_tokens=4,
+                                                         ignore_eos=True))
+    assert len(out) == 2
+
+
+@pytest.mark.gpu
+def test_decode_graph_replays_equal_eager(mixed_model):
+    """Captured decode steps replayed several times, with eager work between
+    the replays, against the same steps run eagerly."""
+    target = ("cuda", "float32")
+    cfg, tensors, path = mixed_model(target)
+    toks = {r: tokens_for(n, cfg["vocab"], 50 + i) for i, (r, n) in enumerate(
+        {"a": 30, "b": 12, "c": 19, "d": 9, "e": 25, "f": 14, "g": 11, "h": 21}.items())}
+    results = []
+    for eager in (True, False):
+        device, dtype = target
+        eng = LLMEngine(EngineConfig(model=path, device=device, dtype=dtype, max_num_seqs=8,
+                                     max_model_len=256, num_kv_blocks=32, enforce_eager=eager))
+        assert eng.runner.use_graphs == (not eager)
+        rows = []
+        eng.replay_step([{"id": r, "tokens": t[:-8], "want": []} for r, t in toks.items()])
+        for k in range(8, 0, -1):
+            rows.append(eng.replay_step(
+                [{"id": r, "tokens": [t[len(t) - k]], "want": [0]} for r, t in toks.items()]))
+            torch.cuda.synchronize()
+        results.append(torch.cat(rows))
+    assert (results[0] - results[1]).abs().max() < 2e-4
+    want = torch.cat([torch.stack([oracle_logits(cfg, tensors, t)[len(t) - k] for t in toks.values()])
+                      for k in range(8, 0, -1)])
+    assert_close(results[1], want, target, "graph replays")
+
+
+def test_trace_runner_cli(tmp_path, mixed_model):
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    import numpy as np
+
+    cfg, tensors, path = mixed_model(("cpu", "float32"))
+    toks = tokens_for(20, cfg["vocab"], 60)
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": toks[:13], "want": [0, 12]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": toks[13:15], "want": []}], "end": []},
+        {"step": 2, "entries": [{"id": "a", "tokens": toks[15:], "want": [4]}], "end": ["a"]},
+    ]
+    out = tmp_path / "out"
+    root = Path(__file__).resolve().parent.parent
+    proc = subprocess.run(
+        [sys.executable, str(root / "bin" / "trace_run"), "--model", path, "--dtype", "float32",
+         "--out", str(out), "--max-tokens", "64"],
+        input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True,
+        timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [ln for ln in proc.stdout.splitlines() if ln.startswith("done")] == \
+        ["done 0", "done 1", "done 2"]
+    want = oracle_logits(cfg, tensors, toks)
+    a = torch.from_numpy(np.fromfile(out / "0.f32", dtype="<f4").reshape(2, -1).copy())
+    b = torch.from_numpy(np.fromfile(out / "2.f32", dtype="<f4").reshape(1, -1).copy())
+    assert not (out / "1.f32").exists()
+    assert_close(torch.cat([a, b]), want[[0, 12, 19]], ("cpu", "float32"), "trace runner")
