@@ -44,7 +44,8 @@ def compare_hybrid(args) -> None:
     models = args.compare_models.split(",")
     batch, prompt_len = min(args.batch, 64), args.prompt_len
     if not use_gpu:
-        tiny = ["tiny-muvetar", "tiny-kosalorn"] if args.compare_muvetar else \
+        tiny = ["tiny-tefudra", "tiny-muvetar"] if args.compare_tefudra else \
+            ["tiny-muvetar", "tiny-kosalorn"] if args.compare_muvetar else \
             ["tiny-kosalorn"] if args.compare_kosalorn else []
         models, batch, prompt_len = tiny + ["tiny-kakovik", "tiny-llama"], 4, 48
     for name in models:
@@ -143,14 +144,21 @@ def main() -> None:
                         "(minGRU, selective scan beside attention, softmax-routed experts) "
                         "beside the Kosalorn expert-mixture preset and the Llama presets of "
                         "equal layer sizes")
+    parser.add_argument("--compare-tefudra", action="store_true",
+                        help="the same comparison for the Tefudra presets (sink attention, "
+                        "capped attention beside an mLSTM matrix memory, routed GELU experts) "
+                        "beside the Kakovik, Muvetar and Llama presets of equal layer sizes")
     args = parser.parse_args()
+    if args.compare_models is None and args.compare_tefudra:
+        args.compare_models = ("tefudra-1b,tefudra-1b-moe,kakovik-1b,muvetar-1b,llama-3.2-1b,"
+                               "tefudra-3b,kakovik-3b,llama-3.2-3b")
     if args.compare_models is None and args.compare_muvetar:
         args.compare_models = "muvetar-1b,kosalorn-1b-moe,llama-3.2-1b,muvetar-3b,kosalorn-3b,llama-3.2-3b"
     if args.compare_models is None:
         args.compare_models = (
             "kosalorn-1b,kosalorn-1b-moe,kakovik-1b,llama-3.2-1b,kosalorn-3b,kakovik-3b,llama-3.2-3b"
             if args.compare_kosalorn else "kakovik-1b,llama-3.2-1b,kakovik-3b,llama-3.2-3b")
-    if args.compare_hybrid or args.compare_kosalorn or args.compare_muvetar:
+    if args.compare_hybrid or args.compare_kosalorn or args.compare_muvetar or args.compare_tefudra:
         compare_hybrid(args)
         return
 
