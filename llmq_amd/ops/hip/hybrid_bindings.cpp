@@ -82,16 +82,20 @@ void sandwich_norm_res32(at::Tensor x, at::Tensor residual, at::Tensor w_post, a
   if (rows == 0) return;
   if (x.scalar_type() == at::kBFloat16 && hidden % 8 == 0 && hidden <= 4 * 2048) {
     using bf = __hip_bfloat16;
-    auto launch = [&]<int CH>() {
-      hipLaunchKernelGGL(sandwich_norm_res32_vec_kernel<CH>, dim3(rows), dim3(256), 0, hy_stream(),
-                         reinterpret_cast<bf*>(x.data_ptr()), residual.data_ptr<float>(),
+    auto launch = [&]<int CH, bool PER_WAVE>() {
+      const long blocks = PER_WAVE ? (rows + 3) / 4 : rows;
+      hipLaunchKernelGGL((sandwich_norm_res32_vec_kernel<CH, PER_WAVE>), dim3(blocks), dim3(256), 0,
+                         hy_stream(), reinterpret_cast<bf*>(x.data_ptr()), residual.data_ptr<float>(),
                          reinterpret_cast<const bf*>(w_post.data_ptr()),
                          reinterpret_cast<const bf*>(w_pre.data_ptr()), hidden, (float)eps,
-                         (float)offset, groups);
+                         (float)offset, groups, rows);
     };
-    if (hidden <= 2048) launch.template operator()<1>();
-    else if (hidden <= 4096) launch.template operator()<2>();
-    else launch.template operator()<4>();
+    // short rows (and the parts of rows normed in groups): a wave per row
+    if (hidden <= 512) launch.template operator()<1, true>();
+    else if (hidden <= 1024) launch.template operator()<2, true>();
+    else if (hidden <= 2048) launch.template operator()<1, false>();
+    else if (hidden <= 4096) launch.template operator()<2, false>();
+    else launch.template operator()<4, false>();
     return;
   }
   hy_dispatch(x, "sandwich_norm_res32", [&]<typename T>() {
@@ -1155,16 +1159,28 @@ void qkv_norm_rope_cache(at::Tensor q, at::Tensor k, const std::optional<at::Ten
     TORCH_CHECK(DV % 2 == 0, "rotated values need an even size");
     v_table = table_ptr(v_inv_freq, DV);
   }
-  TORCH_CHECK(rot_dims <= 2 * 64 * kRopePairs && D - rot_dims <= 64 * kRopeTail &&
-              DV <= 64 * kRopeTail && (!v_table || DV <= 2 * 64 * kRopePairs),
+  // lanes per head vector: the fewest that hold its pairs and unrotated channels
+  const int max_half = std::max<int>(rot_dims / 2, v_table ? DV / 2 : 0);
+  const int max_tail = std::max<int>(D - rot_dims, (v_opt.has_value() && !v_table) ? DV : 0);
+  // bf16 vectors made of whole 16-byte granules: a granule of each half and
+  // one of the rest per lane
+  auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
+  const bool vec = dt == at::kBFloat16 && D % 8 == 0 && DV % 8 == 0 && rot_dims % 16 == 0 &&
+                   (!v_table || DV % 16 == 0) && q.stride(0) % 8 == 0 && k.stride(0) % 8 == 0 &&
+                   v_stride % 8 == 0 && aligned(q.data_ptr()) && aligned(k.data_ptr()) &&
+                   aligned(v_ptr) && aligned(qw) && aligned(kw);
+  const int per_pair = vec ? 8 : kRopePairs, per_tail = vec ? 8 : kRopeTail;
+  int LG = vec ? 1 : 8;
+  while (LG < 64 && (max_half > LG * per_pair || max_tail > LG * per_tail)) LG *= 2;
+  TORCH_CHECK(max_half <= LG * per_pair && max_tail <= LG * per_tail,
               "head size beyond what a wave holds in registers");
   TORCH_CHECK(positions.scalar_type() == at::kLong && positions.is_contiguous() &&
               positions.numel() == T_ && positions.is_cuda());
   TORCH_CHECK(slots.scalar_type() == at::kLong && slots.is_contiguous() && slots.numel() == T_ &&
               slots.is_cuda());
   const size_t lds = sizeof(float) * (size_t)(rot_dims + DV);
-  hy_dispatch(q, "qkv_norm_rope_cache", [&]<typename T>() {
-    hipLaunchKernelGGL(qkv_norm_rope_cache_kernel<T>, dim3(T_), dim3(256), lds, hy_stream(),
+  auto launch = [&]<typename T, bool VEC>() {
+    hipLaunchKernelGGL((qkv_norm_rope_cache_kernel<T, VEC>), dim3(T_), dim3(256), lds, hy_stream(),
                        reinterpret_cast<T*>(q.data_ptr()), q.stride(0),
                        reinterpret_cast<const T*>(k.data_ptr()), k.stride(0),
                        reinterpret_cast<const T*>(v_ptr), v_stride,
@@ -1172,8 +1188,10 @@ void qkv_norm_rope_cache(at::Tensor q, at::Tensor k, const std::optional<at::Ten
                        (int)rot_dims, v_table, positions.data_ptr<long>(),
                        reinterpret_cast<T*>(k_cache.data_ptr()),
                        reinterpret_cast<T*>(v_cache.data_ptr()), slots.data_ptr<long>(), H, G, D, DV,
-                       bs, (float)eps, (int)v_unit_norm);
-  });
+                       bs, (float)eps, (int)v_unit_norm, LG);
+  };
+  if (vec) launch.template operator()<__hip_bfloat16, true>();
+  else hy_dispatch(q, "qkv_norm_rope_cache", [&]<typename T>() { launch.template operator()<T, false>(); });
 }
 
 void rotate_heads(at::Tensor x, at::Tensor positions, at::Tensor inv_freq, bool inverse) {

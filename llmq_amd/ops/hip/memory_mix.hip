@@ -11,10 +11,12 @@
 #include "common.h"
 
 // ------------------------------------------- q / k / v before the attention --
-// One workgroup per token, one wave per head vector at a time. A head vector
-// of n channels whose first rd are rotated in pairs (i, i + rd/2) is held by a
-// wave as up to kRopePairs pairs and kRopeTail unrotated channels per lane, so
-// norm and rotation need no exchange beyond the wave's sum of squares.
+// One workgroup per token. A head vector of n channels whose first rd are
+// rotated in pairs (i, i + rd/2) belongs to a team of LG adjacent lanes (LG a
+// power of two chosen by the host: the fewest lanes that hold the vector as up
+// to kRopePairs pairs and kRopeTail unrotated channels each), so a wave works
+// on 64 / LG heads at once and norm and rotation need no exchange beyond the
+// team's sum of squares.
 //   q [T, H, D] (rows strided): optional RMSNorm x weight, rotation, in place;
 //   k [T, G, D]: the same, into the key cache; with v == null its raw values
 //     go to the value cache (values = keys as projected);
@@ -22,19 +24,20 @@
 //     all DV channels with a table of its own, into the value cache.
 // cos/sin of a token's angles (position * inv_freq[i], fp32, sincosf) are
 // computed once per workgroup into LDS.
-constexpr int kRopePairs = 4;    // 64 * 4 pairs: rotated widths up to 512
-constexpr int kRopeTail = 8;     // 64 * 8 unrotated channels
+constexpr int kRopePairs = 4;
+constexpr int kRopeTail = 8;
 
 template <typename T>
 DEVINL void norm_rope_vector(const T* __restrict__ src, int n, int rd, const T* __restrict__ weight,
-                             bool unit_norm, float eps, const float* __restrict__ cs, int lane,
-                             T* __restrict__ dst, T* __restrict__ raw_dst) {
-  const int half = rd / 2;
+                             bool unit_norm, float eps, const float* __restrict__ cs, int sub,
+                             int LG, bool active, T* __restrict__ dst, T* __restrict__ raw_dst) {
+  const int half = active ? rd / 2 : 0;
+  if (!active) n = 0;
   float u[kRopePairs], v[kRopePairs], t[kRopeTail];
   float ss = 0.f;
 #pragma unroll
   for (int j = 0; j < kRopePairs; ++j) {
-    const int i = lane + 64 * j;
+    const int i = sub + LG * j;
     u[j] = v[j] = 0.f;
     if (i < half) {
       u[j] = to_f32(src[i]);
@@ -48,7 +51,7 @@ DEVINL void norm_rope_vector(const T* __restrict__ src, int n, int rd, const T* 
   }
 #pragma unroll
   for (int j = 0; j < kRopeTail; ++j) {
-    const int c = rd + lane + 64 * j;
+    const int c = rd + sub + LG * j;
     t[j] = 0.f;
     if (c < n) {
       t[j] = to_f32(src[c]);
@@ -57,13 +60,13 @@ DEVINL void norm_rope_vector(const T* __restrict__ src, int n, int rd, const T* 
     ss += t[j] * t[j];
   }
   float inv = 1.f;
-  if (weight || unit_norm) {
-    ss = wave_reduce_sum(ss);
-    inv = 1.0f / sqrtf(ss / n + eps);
+  if (weight || unit_norm) {         // uniform over the wave: every lane takes part
+    for (int off = LG >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, WAVE);
+    inv = 1.0f / sqrtf(ss / max(n, 1) + eps);
   }
 #pragma unroll
   for (int j = 0; j < kRopePairs; ++j) {
-    const int i = lane + 64 * j;
+    const int i = sub + LG * j;
     if (i < half) {
       float a = u[j] * inv, b = v[j] * inv;
       if (weight) {
@@ -77,7 +80,7 @@ DEVINL void norm_rope_vector(const T* __restrict__ src, int n, int rd, const T* 
   }
 #pragma unroll
   for (int j = 0; j < kRopeTail; ++j) {
-    const int c = rd + lane + 64 * j;
+    const int c = rd + sub + LG * j;
     if (c < n) {
       float a = t[j] * inv;
       if (weight) a *= to_f32(weight[c]);
@@ -86,7 +89,91 @@ DEVINL void norm_rope_vector(const T* __restrict__ src, int n, int rd, const T* 
   }
 }
 
-template <typename T>
+// The 16-byte form for bf16 vectors whose halves and unrotated rest are whole
+// granules of 8: a lane holds at most one granule of each half (8 pairs) and
+// one granule of the rest, so a team is as small as a vector has granule
+// pairs and every access is one 16-byte load or store.
+DEVINL void norm_rope_vec8(const __hip_bfloat16* __restrict__ src, int n, int rd,
+                           const __hip_bfloat16* __restrict__ weight, bool unit_norm, float eps,
+                           const float* __restrict__ cs, int sub, int LG, bool active,
+                           __hip_bfloat16* __restrict__ dst, __hip_bfloat16* __restrict__ raw_dst) {
+  using bf = __hip_bfloat16;
+  const int half = rd / 2;
+  const bool has_pair = active && sub * 8 < half;
+  const bool has_tail = active && rd + sub * 8 < n;
+  float u[8], v[8], t[8];
+  float ss = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) u[e] = v[e] = t[e] = 0.f;
+  if (has_pair) {
+    const Vec8<bf> a = load16(src + sub * 8), b = load16(src + half + sub * 8);
+    if (raw_dst) {
+      store16(raw_dst + sub * 8, a);
+      store16(raw_dst + half + sub * 8, b);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      u[e] = to_f32(a.data[e]);
+      v[e] = to_f32(b.data[e]);
+      ss += u[e] * u[e] + v[e] * v[e];
+    }
+  }
+  if (has_tail) {
+    const Vec8<bf> a = load16(src + rd + sub * 8);
+    if (raw_dst) store16(raw_dst + rd + sub * 8, a);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      t[e] = to_f32(a.data[e]);
+      ss += t[e] * t[e];
+    }
+  }
+  float inv = 1.f;
+  if (weight || unit_norm) {         // uniform over the wave: every lane takes part
+    for (int off = LG >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, WAVE);
+    inv = 1.0f / sqrtf(ss / max(active ? n : 1, 1) + eps);
+  }
+  if (has_pair) {
+    Vec8<bf> wa, wb, oa, ob;
+    if (weight) {
+      wa = load16(weight + sub * 8);
+      wb = load16(weight + half + sub * 8);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float a = u[e] * inv, b = v[e] * inv;
+      if (weight) {
+        a *= to_f32(wa.data[e]);
+        b *= to_f32(wb.data[e]);
+      }
+      const float2 c_s = *reinterpret_cast<const float2*>(cs + 2 * (sub * 8 + e));
+      oa.data[e] = __float2bfloat16(a * c_s.x - b * c_s.y);
+      ob.data[e] = __float2bfloat16(b * c_s.x + a * c_s.y);
+    }
+    store16(dst + sub * 8, oa);
+    store16(dst + half + sub * 8, ob);
+  }
+  if (has_tail) {
+    Vec8<bf> wt, ot;
+    if (weight) wt = load16(weight + rd + sub * 8);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      float a = t[e] * inv;
+      if (weight) a *= to_f32(wt.data[e]);
+      ot.data[e] = __float2bfloat16(a);
+    }
+    store16(dst + rd + sub * 8, ot);
+  }
+}
+
+template <typename T, bool VEC>
+DEVINL void norm_rope_any(const T* __restrict__ src, int n, int rd, const T* __restrict__ weight,
+                          bool unit_norm, float eps, const float* __restrict__ cs, int sub, int LG,
+                          bool active, T* __restrict__ dst, T* __restrict__ raw_dst) {
+  if constexpr (VEC) norm_rope_vec8(src, n, rd, weight, unit_norm, eps, cs, sub, LG, active, dst, raw_dst);
+  else norm_rope_vector<T>(src, n, rd, weight, unit_norm, eps, cs, sub, LG, active, dst, raw_dst);
+}
+
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void qkv_norm_rope_cache_kernel(
     T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
     const T* __restrict__ v, long v_stride,               // null: values = raw keys
@@ -95,8 +182,8 @@ __global__ __launch_bounds__(256) void qkv_norm_rope_cache_kernel(
     const float* __restrict__ v_inv_freq,                 // [DV / 2] or null
     const long* __restrict__ positions, T* __restrict__ k_cache, T* __restrict__ v_cache,
     const long* __restrict__ slots, int H, int G, int D, int DV, int block_size, float eps,
-    int v_unit_norm) {
-  extern __shared__ float cs_smem[];
+    int v_unit_norm, int LG) {
+  extern __shared__ __align__(8) float cs_smem[];
   float* cs = cs_smem;                       // [rot_dims/2][cos, sin]
   float* vcs = cs + rot_dims;                // [DV/2][cos, sin]
   const long tok = blockIdx.x;
@@ -120,23 +207,28 @@ __global__ __launch_bounds__(256) void qkv_norm_rope_cache_kernel(
   const long slot = slots[tok];
   const long blk = slot >= 0 ? slot / block_size : 0;
   const int off = slot >= 0 ? (int)(slot % block_size) : 0;
-  const int items = H + G + (v ? G : 0);
-  for (int it = w; it < items; it += 4) {
-    if (it < H) {
-      T* qh = q + tok * q_stride + (long)it * D;
-      norm_rope_vector<T>(qh, D, rot_dims, q_w, false, eps, cs, lane, qh, nullptr);
-    } else if (it < H + G) {
-      if (slot < 0) continue;
-      const int g = it - H;
-      const long row = (blk * G + g) * block_size + off;
-      norm_rope_vector<T>(k + tok * k_stride + (long)g * D, D, rot_dims, k_w, false, eps, cs,
-                          lane, k_cache + row * D, v ? nullptr : v_cache + row * DV);
-    } else {
-      if (slot < 0) continue;
-      const int g = it - H - G;
-      const long row = (blk * G + g) * block_size + off;
-      norm_rope_vector<T>(v + tok * v_stride + (long)g * DV, DV, v_inv_freq ? DV : 0, nullptr,
-                          v_unit_norm != 0, eps, vcs, lane, v_cache + row * DV, nullptr);
+  const int per_wave = 64 / LG, sub = lane % LG, team = lane / LG;
+  // three passes, each uniform over the wave in what it norms: q, k, v
+  for (int base = w * per_wave; base < H; base += 4 * per_wave) {
+    const int h = base + team;
+    T* qh = q + tok * q_stride + (long)min(h, H - 1) * D;
+    norm_rope_any<T, VEC>(qh, D, rot_dims, q_w, false, eps, cs, sub, LG, h < H, qh, nullptr);
+  }
+  for (int base = w * per_wave; base < G; base += 4 * per_wave) {
+    const int g = base + team;
+    const bool act = g < G && slot >= 0;
+    const long row = (blk * G + min(g, G - 1)) * block_size + off;
+    norm_rope_any<T, VEC>(k + tok * k_stride + (long)min(g, G - 1) * D, D, rot_dims, k_w, false,
+                          eps, cs, sub, LG, act, k_cache + row * D, v ? nullptr : v_cache + row * DV);
+  }
+  if (v) {
+    for (int base = w * per_wave; base < G; base += 4 * per_wave) {
+      const int g = base + team;
+      const bool act = g < G && slot >= 0;
+      const long row = (blk * G + min(g, G - 1)) * block_size + off;
+      norm_rope_any<T, VEC>(v + tok * v_stride + (long)min(g, G - 1) * DV, DV, v_inv_freq ? DV : 0,
+                            nullptr, v_unit_norm != 0, eps, vcs, sub, LG, act, v_cache + row * DV,
+                            nullptr);
     }
   }
 }

@@ -76,14 +76,19 @@ __global__ void sandwich_norm_res32_kernel(T* __restrict__ x, float* __restrict_
 // The same sandwich for bf16 rows of up to CH * 2048 elements, a multiple of
 // 8 wide: every thread keeps its 8-element granules of the updated residual
 // in registers, so x, the residual and the two weights cross memory exactly
-// once, in 16-byte accesses.
-template <int CH>
+// once, in 16-byte accesses. PER_WAVE: a row (or one part of a row normed in
+// groups) of up to CH * 512 elements belongs to one wave, four rows to a
+// workgroup, and the two sums are wave reductions without LDS or barriers.
+template <int CH, bool PER_WAVE>
 __global__ __launch_bounds__(256) void sandwich_norm_res32_vec_kernel(
     __hip_bfloat16* __restrict__ x, float* __restrict__ residual,
     const __hip_bfloat16* __restrict__ w_post, const __hip_bfloat16* __restrict__ w_pre,
-    int hidden, float eps, float offset, int groups) {
+    int hidden, float eps, float offset, int groups, long rows) {
   __shared__ float red[4];
-  const long row = blockIdx.x;
+  constexpr int TEAM = PER_WAVE ? 64 : 256;
+  const int member = PER_WAVE ? (threadIdx.x & 63) : threadIdx.x;
+  const long row = PER_WAVE ? blockIdx.x * 4L + (threadIdx.x >> 6) : blockIdx.x;
+  if (PER_WAVE && row >= rows) return;
   w_post += (row % groups) * hidden;
   w_pre += (row % groups) * hidden;
   __hip_bfloat16* xr = x + row * hidden;
@@ -92,7 +97,7 @@ __global__ __launch_bounds__(256) void sandwich_norm_res32_vec_kernel(
   float ss = 0.f;
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
-    const int i = (c * 256 + threadIdx.x) * 8;
+    const int i = (c * TEAM + member) * 8;
     if (i < hidden) {
       const Vec8<__hip_bfloat16> v = load16(xr + i);
       const float4 ra = *reinterpret_cast<const float4*>(rr + i);
@@ -106,12 +111,12 @@ __global__ __launch_bounds__(256) void sandwich_norm_res32_vec_kernel(
       }
     }
   }
-  ss = block_reduce_sum(ss, red);
+  ss = PER_WAVE ? wave_reduce_sum(ss) : block_reduce_sum(ss, red);
   const float inv1 = 1.0f / sqrtf(ss / hidden + eps);
   float ss2 = 0.f;
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
-    const int i = (c * 256 + threadIdx.x) * 8;
+    const int i = (c * TEAM + member) * 8;
     if (i < hidden) {
       const Vec8<__hip_bfloat16> wv = load16(w_post + i);
 #pragma unroll
@@ -123,11 +128,11 @@ __global__ __launch_bounds__(256) void sandwich_norm_res32_vec_kernel(
       *reinterpret_cast<float4*>(rr + i + 4) = make_float4(rv[c][4], rv[c][5], rv[c][6], rv[c][7]);
     }
   }
-  ss2 = block_reduce_sum(ss2, red);
+  ss2 = PER_WAVE ? wave_reduce_sum(ss2) : block_reduce_sum(ss2, red);
   const float inv2 = 1.0f / sqrtf(ss2 / hidden + eps);
 #pragma unroll
   for (int c = 0; c < CH; ++c) {
-    const int i = (c * 256 + threadIdx.x) * 8;
+    const int i = (c * TEAM + member) * 8;
     if (i < hidden) {
       const Vec8<__hip_bfloat16> wv = load16(w_pre + i);
       Vec8<__hip_bfloat16> ov;

@@ -179,7 +179,7 @@ def tolerance(target):
     """(worst row, mean over rows) of the relative rms error. fp32 is the
     sharp comparison; bf16 rounds every GEMM input and output of a deep
     stack and only has to stay at rounding level."""
-    return (8e-2, 2.5e-2) if target[1] == "bfloat16" else (2e-4, 5e-5)
+    return (1e-1, 4e-2) if target[1] == "bfloat16" else (2e-4, 5e-5)
 
 
 def assert_close(got, want, target, what=""):
@@ -608,6 +608,49 @@ def test_values_rotate_by_their_position_and_back(target):
     assert (q[..., 4:] - q0[..., 4:]).abs().max().item() == 0.0
     n0 = q0.double()[..., :4].pow(2).sum(-1)
     assert ((q.double()[..., :4].pow(2).sum(-1) - n0).abs() / n0).max().item() < 10 * tol
+
+
+@pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("H,G,D,DV,rot,own_v", [(4, 2, 64, 64, 64, True), (6, 2, 128, 128, 64, False),
+                                                (6, 2, 96, 96, 96, True), (3, 1, 40, 24, 16, True),
+                                                (2, 2, 16, 10, 6, True), (5, 1, 136, 136, 32, False)])
+def test_norm_rotate_scatter_op(target, H, G, D, DV, rot, own_v):
+    """The per-token kernel between projections and attention, in both of its
+    uses (per-head q/k norm with values = raw keys; plain q/k with unit-norm
+    rotated values), over head sizes that do and do not fill 16-byte granules,
+    on rows that are column slices of a wider matrix."""
+    from llmq_amd.engine.models.kosalorn import rotary_inv_freq
+
+    device, dtype = dev_dtype(target)
+    g = torch.Generator().manual_seed(D + DV)
+    T, bs, eps, base = 21, 16, 1e-5, 5000.0
+    wide = torch.randn(T, 8 + H * D + G * D + G * DV, generator=g).to(dtype).to(device)
+    q = wide[:, 8:8 + H * D].unflatten(1, (H, D))
+    k = wide[:, 8 + H * D:8 + (H + G) * D].unflatten(1, (G, D))
+    v = wide[:, 8 + (H + G) * D:].unflatten(1, (G, DV)) if own_v else None
+    q0, k0 = q.double().cpu(), k.double().cpu()
+    qw = None if own_v else (torch.randn(D, generator=g) * 0.2 + 1).to(dtype)
+    kw = None if own_v else (torch.randn(D, generator=g) * 0.2 + 1).to(dtype)
+    kc = torch.zeros(3, G, bs, D, dtype=dtype, device=device)
+    vc = torch.zeros(3, G, bs, DV, dtype=dtype, device=device)
+    first = 200                                         # positions away from 0
+    pos = torch.arange(first, first + T, dtype=torch.long, device=device)
+    slots = torch.arange(5, 5 + T, dtype=torch.long, device=device)
+    ops.qkv_norm_rope_cache(
+        q, k, v, None if qw is None else qw.to(device), None if kw is None else kw.to(device),
+        rotary_inv_freq(base, rot).to(device), rot, pos, kc, vc, slots, eps, v_unit_norm=own_v,
+        v_inv_freq=rotary_inv_freq(base, DV).to(device) if own_v else None)
+    want_q = q0 if qw is None else oracle.rms(q0, eps) * qw.double()
+    want_k = k0 if kw is None else oracle.rms(k0, eps) * kw.double()
+    want_q = oracle.rotate_half(want_q, first, base, rot)
+    want_k = oracle.rotate_half(want_k, first, base, rot)
+    want_v = oracle.rotate_half(oracle.rms(v.double().cpu(), eps), first, base, DV) if own_v else k0
+    got_k = kc.permute(0, 2, 1, 3).reshape(-1, G, D)[5:5 + T].double().cpu()
+    got_v = vc.permute(0, 2, 1, 3).reshape(-1, G, DV)[5:5 + T].double().cpu()
+    tol = 2e-2 if dtype == torch.bfloat16 else 5e-5      # fp32 angles at positions in the hundreds
+    for got, want in ((q.double().cpu(), want_q), (got_k, want_k), (got_v, want_v)):
+        assert (got - want).abs().max().item() < tol * want.abs().max().item()
+    assert float(kc.reshape(-1, G, bs, D)[0, :, :5].abs().max()) == 0.0   # rows before the slots
 
 
 # ------------------------------------------------------ ops against oracle --
