@@ -1309,6 +1309,20 @@ void dual_norm_mean(at::Tensor out, at::Tensor a, at::Tensor w_a, at::Tensor b, 
   TORCH_CHECK(b.scalar_type() == dt && out.scalar_type() == dt && w_a.scalar_type() == dt &&
               w_b.scalar_type() == dt && w_a.is_contiguous() && w_b.is_contiguous() &&
               w_a.numel() == W && w_b.numel() == W);
+  if (dt == at::kBFloat16 && W % 8 == 0 && W <= 4 * 2048) {
+    using bf = __hip_bfloat16;
+    auto launch = [&]<int CH>() {
+      hipLaunchKernelGGL(dual_norm_mean_vec_kernel<CH>, dim3(rows), dim3(256), 0, hy_stream(),
+                         reinterpret_cast<bf*>(out.data_ptr()), reinterpret_cast<const bf*>(a.data_ptr()),
+                         reinterpret_cast<const bf*>(w_a.data_ptr()),
+                         reinterpret_cast<const bf*>(b.data_ptr()),
+                         reinterpret_cast<const bf*>(w_b.data_ptr()), W, (float)eps);
+    };
+    if (W <= 2048) launch.template operator()<1>();
+    else if (W <= 4096) launch.template operator()<2>();
+    else launch.template operator()<4>();
+    return;
+  }
   hy_dispatch(a, "dual_norm_mean", [&]<typename T>() {
     hipLaunchKernelGGL(dual_norm_mean_kernel<T>, dim3(rows), dim3(256), 0, hy_stream(),
                        reinterpret_cast<T*>(out.data_ptr()), reinterpret_cast<const T*>(a.data_ptr()),

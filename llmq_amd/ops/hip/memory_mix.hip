@@ -368,6 +368,52 @@ __global__ __launch_bounds__(256) void dual_norm_mean_kernel(
                                                  to_f32(br[i]) * ib * to_f32(w_b[i])));
 }
 
+// The same for bf16 rows of up to CH * 2048 elements, a multiple of 8 wide:
+// both rows stay in registers between the sums and the result, every access
+// is 16 bytes.
+template <int CH>
+__global__ __launch_bounds__(256) void dual_norm_mean_vec_kernel(
+    __hip_bfloat16* __restrict__ out, const __hip_bfloat16* __restrict__ a,
+    const __hip_bfloat16* __restrict__ w_a, const __hip_bfloat16* __restrict__ b,
+    const __hip_bfloat16* __restrict__ w_b, int hidden, float eps) {
+  using bf = __hip_bfloat16;
+  __shared__ float red[4];
+  const long row = blockIdx.x;
+  float av[CH][8], bv[CH][8];
+  float sa = 0.f, sb = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 8;
+    if (i < hidden) {
+      const Vec8<bf> x = load16(a + row * hidden + i), y = load16(b + row * hidden + i);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        av[c][j] = to_f32(x.data[j]);
+        bv[c][j] = to_f32(y.data[j]);
+        sa += av[c][j] * av[c][j];
+        sb += bv[c][j] * bv[c][j];
+      }
+    }
+  }
+  sa = block_reduce_sum(sa, red);
+  __syncthreads();
+  sb = block_reduce_sum(sb, red);
+  const float ia = 0.5f / sqrtf(sa / hidden + eps), ib = 0.5f / sqrtf(sb / hidden + eps);
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int i = (c * 256 + threadIdx.x) * 8;
+    if (i < hidden) {
+      const Vec8<bf> wa = load16(w_a + i), wb = load16(w_b + i);
+      Vec8<bf> o;
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        o.data[j] = __float2bfloat16(av[c][j] * ia * to_f32(wa.data[j]) +
+                                     bv[c][j] * ib * to_f32(wb.data[j]));
+      store16(out + row * hidden + i, o);
+    }
+  }
+}
+
 // ------------------------------------------------------ ungated activations --
 constexpr int kActRelu2 = 0;
 constexpr int kActGeluErf = 1;
