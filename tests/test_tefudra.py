@@ -611,8 +611,8 @@ def test_values_rotate_by_their_position_and_back(target):
 
 
 @pytest.mark.parametrize("target", DEVICES)
-@pytest.mark.parametrize("H,G,D,DV,rot,own_v", [(4, 2, 64, 64, 64, True), (6, 2, 128, 128, 64, False),
-                                                (6, 2, 96, 96, 96, True), (3, 1, 40, 24, 16, True),
+@pytest.mark.parametrize("H,G,D,DV,rot,own_v", [(4, 2, 64, 64, 64, True), (8, 4, 128, 128, 32, False),
+                                                (4, 1, 80, 80, 80, True), (3, 1, 40, 24, 16, True),
                                                 (2, 2, 16, 10, 6, True), (5, 1, 136, 136, 32, False)])
 def test_norm_rotate_scatter_op(target, H, G, D, DV, rot, own_v):
     """The per-token kernel between projections and attention, in both of its
@@ -761,7 +761,7 @@ def test_expert_mixture_with_identity_experts(target, W, F, E, ident, top, T):
 
 
 @pytest.mark.parametrize("target", DEVICES)
-@pytest.mark.parametrize("W,groups", [(48, 3), (27, 3), (2048, 4), (2056, 1), (192, 4)])
+@pytest.mark.parametrize("W,groups", [(48, 3), (27, 3), (2048, 4), (2056, 1), (256, 8), (3072, 4)])
 def test_grouped_norms_joins_and_activations(target, W, groups):
     device, dtype = dev_dtype(target)
     g = torch.Generator().manual_seed(W)
