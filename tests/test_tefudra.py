@@ -360,6 +360,51 @@ def test_expert_choice_in_the_model(tmp_path, target, experts, identity, top):
                  f"{experts}+{identity} experts, top {top}")
 
 
+@pytest.mark.parametrize("target", DEVICES)
+def test_wider_model_with_other_sizes(tmp_path, target):
+    """Head sizes that fill the kernels' 16-byte paths and the matrix cores,
+    five norm groups, windows that several portions and decoded tokens pass,
+    a pair layer on shared weights; whole, cut and beside another request."""
+    route = target[1] != "bfloat16"
+    moe = moe_cfg(experts=9, identity=3, top=2, ff=40, shared=56) if route else \
+        moe_cfg(experts=3, identity=1, top=4, ff=40, shared=56)
+    layers = [
+        attn(heads=8, kv_heads=4, dim=48, rot_dims=32, base=50000.0, size=50, keep=9, scale=0.15,
+             mlp=dense(200)),
+        par(heads=6, kv_heads=2, dim=40, vdim=56, rot_dims=16, base=3000.0, size=33, scale=0.2,
+            softcap=12.0, conv=5, mheads=4, mdim=24, mvdim=40, gate_cap=12.0, mlp=moe),
+        par(heads=6, kv_heads=2, dim=40, vdim=56, rot_dims=16, base=3000.0, size=33, scale=0.2,
+            softcap=12.0, conv=5, mheads=4, mdim=24, mvdim=40, gate_cap=12.0, mlp=moe, weights_of=1),
+        attn(heads=3, kv_heads=1, dim=64, rot_dims=64, size=64, keep=1, scale=0.125, mlp=None),
+    ]
+    cfg = make_config(layers, width=160, vocab=300, eps=1e-6, groups=5)
+    tensors = make_tensors(cfg, seed=21)
+    path = write_checkpoint(tmp_path / "m", cfg, tensors)
+    t64 = f64(tensors)
+    a, b = tokens_for(200, 300, 80), tokens_for(90, 300, 81)
+    want_a, want_b = oracle.forward(cfg, t64, a), oracle.forward(cfg, t64, b)
+    eng = make_engine(path, target, blocks=24)
+    assert_close(replay(eng, "w", a, [200]), want_a, target, "whole")
+    assert_close(replay(eng, "c", a, [63, 2, 65, 1, 1, 1, 1, 30, 36]), want_a, target, "cut")
+    # b's portions beside a's single tokens, then b's single tokens beside a's portion
+    got_a = [eng.replay_step([{"id": "a", "tokens": a[:120], "want": list(range(120))}])]
+    got_b = []
+    for k in range(40):
+        out = eng.replay_step([{"id": "a", "tokens": [a[120 + k]], "want": [0]},
+                               {"id": "b", "tokens": b[2 * k:2 * k + 2], "want": [0, 1]}])
+        got_a.append(out[:1])
+        got_b.append(out[1:])
+    out = eng.replay_step([{"id": "b", "tokens": [b[80]], "want": [0]},
+                           {"id": "a", "tokens": a[160:], "want": list(range(40))}])
+    got_b.append(out[:1])
+    got_a.append(out[1:])
+    got_b.append(eng.replay_step([{"id": "b", "tokens": b[81:], "want": list(range(9))}],
+                                 end=["a", "b"]))
+    assert_close(torch.cat(got_a), want_a, target, "a in the batch")
+    assert_close(torch.cat(got_b), want_b, target, "b in the batch")
+    assert eng.allocator.num_free == 24
+
+
 # ------------------------------------------- schedules: cuts, batches, reuse --
 
 @pytest.mark.parametrize("target", DEVICES)
