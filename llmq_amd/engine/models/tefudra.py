@@ -352,7 +352,7 @@ class TefudraLM:
                             act="gelu_erf", weight_output=True, identity=e.identity)
         if e.shared_ff:
             mid = ops.unary_act(F.linear(h, lw.t["s_up"]), "gelu_erf")
-            y = y + F.linear(mid, lw.t["s_down"])
+            y = torch.addmm(y, mid, lw.t["s_down"].t())     # the join rides on the GEMM
         return y
 
     # -- forward ---------------------------------------------------------

@@ -270,12 +270,13 @@ DEVINL float dist_bias(const float* __restrict__ bias, int bias_len, int mode, i
   return bias[(long)h * bias_len + min(d, bias_len - 1)];
 }
 
-// Score cap: c * tanh(s / c). FAST (bf16 models): through the hardware
-// exponential, 1 - 2 / (e^(2x) + 1); fp32 models: tanhf.
+// Score cap: c * tanh(s / c), with 1 / c computed once per kernel. FAST (bf16
+// models): through the hardware exponential and reciprocal,
+// 1 - 2 / (e^(2x) + 1); fp32 models: tanhf.
 template <bool FAST>
-DEVINL float cap_score(float s, float cap) {
-  const float x = s / cap;
-  return cap * (FAST ? 1.0f - 2.0f / (__expf(2.0f * x) + 1.0f) : tanhf(x));
+DEVINL float cap_score(float s, float cap, float inv_cap) {
+  const float x = s * inv_cap;
+  return cap * (FAST ? 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * x) + 1.0f) : tanhf(x));
 }
 
 // Kept first tokens (window mask only): besides its window a query sees every
@@ -343,6 +344,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
   const int* bt = block_tables + (long)b * bt_stride;
   const int lo = mask_first_key(pos0, span, mask_mode);
   const int first_end = min(keep_first, lo);   // keys [0, first_end): kept, before every window
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
   for (int kt = first_end > 0 ? 0 : lo; kt <= pos_last;) {
     const bool in_first = kt < first_end;
     const int kt_next = (in_first && kt + kAttnKT >= first_end) ? lo : kt + kAttnKT;
@@ -382,7 +384,7 @@ __global__ __launch_bounds__(256) void chunk_bias_attn_prefill_kernel(
       const int i = pos0 + w * 4 + r;
       const bool vis = lane < nk && (w * 4 + r) < rows && key <= i &&
                        (key >= mask_first_key(i, span, mask_mode) || key < keep_first);
-      const float sr = softcap > 0.f ? cap_score<sizeof(T) == 2>(s[r], softcap) : s[r];
+      const float sr = softcap > 0.f ? cap_score<sizeof(T) == 2>(s[r], softcap, inv_cap) : s[r];
       const float sc = !vis ? -INFINITY
           : bias ? sr + dist_bias<sizeof(T) == 2>(bias, bias_len, bias_mode, h, i - key) : sr;
       const float tmax = wave_reduce_max(sc);
@@ -584,6 +586,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
   // kept first tokens (never together with key splits): their tiles come first
   const int win0 = kt0;
   const int first_end = min(keep_first, win0);
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
   if (first_end > 0) kt0 = 0;
   if (kt0 <= key_end) fetch(kt0);
   for (int kt = kt0; kt <= key_end;) {
@@ -639,7 +642,7 @@ __global__ __launch_bounds__(256, 2) void chunk_bias_attn_prefill_mfma_kernel(
           const bool vis = key <= irow[reg] &&
               (in_first ? key < first_end : (key >= lorow[reg] || key < keep_first));
           float sc = s[ct][reg] * scale;
-          if (softcap > 0.f) sc = cap_score<true>(sc, softcap);
+          if (softcap > 0.f) sc = cap_score<true>(sc, softcap, inv_cap);
           sv[ct] = vis ? sc + brow[-ct * 16] : -INFINITY;
           tmax = fmaxf(tmax, sv[ct]);
         }
@@ -817,6 +820,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
   }
   // tiles: first the kept keys below the window, then the window's
   const int first_end = min(keep_first, lo);
+  const float inv_cap = softcap > 0.f ? 1.0f / softcap : 0.f;
   const int n_first = (first_end + 63) / 64;
   const int n_tiles = n_first + (i - lo) / 64 + 1;
   for (int tile = w; tile < n_tiles; tile += NW) {
@@ -858,7 +862,7 @@ __global__ __launch_bounds__(64 * kDecWaves) void chunk_bias_attn_decode_kernel(
       }
 #pragma unroll
       for (int hh = 0; hh < HPW; ++hh) {
-        const float sr = softcap > 0.f ? cap_score<sizeof(T) == 2>(s[hh], softcap) : s[hh];
+        const float sr = softcap > 0.f ? cap_score<sizeof(T) == 2>(s[hh], softcap, inv_cap) : s[hh];
         sc[hh] = bias ? sr + dist_bias<sizeof(T) == 2>(bias, bias_len, bias_mode, h0 + hh, i - key)
                       : sr;
       }
