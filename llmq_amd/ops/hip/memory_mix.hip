@@ -4,7 +4,7 @@
 // the turn-back of attended values, the gate walk and the read-out of an mLSTM,
 // the average of two normed mixer outputs, and ungated activations.
 //
-// Numerics contract: activations arrive in the model dtype T (bf16 or fp32);
+// Numerics shared by every kernel here: activations arrive in the model dtype T (bf16 or fp32);
 // norms, angles, gates, running maxima and denominators are fp32 with the
 // accurate library functions and rounded to T once, on store.
 

@@ -313,9 +313,11 @@ def test_config_reader_takes_everything_from_config(tmp_path):
     ([attn(mlp=moe_cfg(experts=3, identity=0, top=3, shared=None))], {}),
     ([attn(mlp=moe_cfg(experts=1, identity=1, top=2))], {}),
     ([par(mlp=None), par(mlp=None, weights_of=0), attn(mlp=None), attn(mlp=None, weights_of=2)], {}),
+    ([attn(weights_of=2), par(weights_of=3), attn(), par()], {}),     # owners after their users
+    ([attn(rot_dims=0, mlp=None), par(rot_dims=0, mlp=None)], {}),
 ], ids=["sink", "sink-plain-window", "sink-wide-window", "sink-keep-beyond-window", "pair",
         "pair-loose-cap-no-conv", "pair-ones", "pair-wide", "dense", "moe-all", "moe-no-identity",
-        "moe-single", "shared-weights"])
+        "moe-single", "shared-weights", "shared-weights-forward", "no-rotation"])
 def test_mechanism_alone(tmp_path, target, layers, kw):
     cfg = make_config(layers, **kw)
     tensors = make_tensors(cfg, seed=3)
