@@ -685,8 +685,8 @@ def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False, act: str = "s
         _use_hybrid(h)
         F_ = down.shape[2]
         plain = gated and not identity
-        if (T * top >= MOE_GROUP_MIN_ROWS and E * T <= MOE_DENSE_MAX_PAIRS) if plain \
-                else (sync_free or E * T <= MOE_DENSE_MAX_PAIRS):
+        if T * top >= MOE_GROUP_MIN_ROWS and (E * T <= MOE_DENSE_MAX_PAIRS or
+                                              (sync_free and not plain)):
             wd = torch.zeros(T, E + identity, dtype=torch.float32, device=h.device)
             wd.scatter_(1, idx.long(), w)
             if weight_output:
@@ -702,6 +702,21 @@ def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False, act: str = "s
                 yk = torch.cat([yk, h.unsqueeze(0)], dim=0)
                 wd = torch.cat([wd[:, :E], wd[:, E:].sum(dim=1, keepdim=True)], dim=1)
             _HY.moe_combine(y, yk, wd if weight_output else None)
+            return y
+        if not plain:
+            # few rows of ungated experts: the matrix-vector kernels read only
+            # the chosen experts; an identity expert's row runs on a stand-in
+            # expert with weight 0 and the token itself joins afterwards
+            hmid = torch.empty(T * top, F_, dtype=h.dtype, device=h.device)
+            real = idx < E
+            w_real = torch.where(real, w, torch.zeros_like(w))
+            _HY.moe_gate_up_gemv(hmid, h, idx, None if weight_output else w, gate_up,
+                                 _MOE_PLAIN_ACTS[act], 0.0)
+            y = torch.empty_like(h)
+            _HY.moe_down_gemv(y, hmid, idx, down, w_real if weight_output else None)
+            if identity:
+                w_id = (w - w_real).sum(dim=1, keepdim=True)
+                y = torch.addcmul(y.float(), h.float(), w_id).to(h.dtype)
             return y
         if plain:
             act_mode = _MOE_ACTS[act]
@@ -752,6 +767,7 @@ def moe_experts(h, idx, w, gate_up, down, sync_free: bool = False, act: str = "s
 
 
 _MOE_ACTS = {"silu": 0, "clamp_swish": 1}
+_MOE_PLAIN_ACTS = {"gelu_erf": 2, "relu2": 3}
 
 
 # ---- scan hybrids: elementwise gated recurrences, selective scans beside

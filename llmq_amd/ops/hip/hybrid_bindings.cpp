@@ -620,11 +620,12 @@ void moe_gate_up_gemv(at::Tensor hmid, at::Tensor h, at::Tensor idx,
                       double limit) {
   HY_GPU(h);
   TORCH_CHECK(h.dim() == 2 && h.is_contiguous() && gate_up.dim() == 3 && gate_up.is_contiguous());
-  TORCH_CHECK(gate_up.size(1) % 2 == 0 && gate_up.size(2) == h.size(1));
-  const MoeDims m = moe_check(idx, h.size(1), gate_up.size(1) / 2, gate_up.size(0));
+  TORCH_CHECK(act >= kMoeActSilu && act <= kMoeActRelu2, "unknown expert activation");
+  const bool gated = act < kMoeActGeluErf;      // ungated experts: gate_up is [E, F, W]
+  TORCH_CHECK((!gated || gate_up.size(1) % 2 == 0) && gate_up.size(2) == h.size(1));
+  const MoeDims m = moe_check(idx, h.size(1), gate_up.size(1) / (gated ? 2 : 1), gate_up.size(0));
   if (m.T == 0) return;
   TORCH_CHECK(idx.size(0) == h.size(0));
-  TORCH_CHECK(act == kMoeActSilu || act == kMoeActClampSwish, "unknown expert activation");
   const float* wp = nullptr;
   if (w.has_value()) {
     TORCH_CHECK(w->scalar_type() == at::kFloat && w->is_contiguous() && w->sizes() == idx.sizes() &&

@@ -250,8 +250,19 @@ constexpr int kMoeRowsPerWave = 4;
 
 // What an expert does between its two projections. Plain: silu(g) * u.
 // Clamped: g = min(g, limit), u = clamp(u, +-limit), g * sigmoid(1.702 g) * (u + 1).
+// Ungated experts (one projection, [E, F, W]): the exact GELU, or relu(.)^2.
 constexpr int kMoeActSilu = 0;
 constexpr int kMoeActClampSwish = 1;
+constexpr int kMoeActGeluErf = 2;
+constexpr int kMoeActRelu2 = 3;
+
+DEVINL float moe_plain_act(float u, int act) {
+  if (act == kMoeActRelu2) {
+    const float r = fmaxf(u, 0.f);
+    return r * r;
+  }
+  return 0.5f * u * (1.0f + erff(u * 0.70710678118654752f));
+}
 
 DEVINL float moe_gated_act(float g, float u, int act, float limit) {
   if (act == kMoeActClampSwish) {
@@ -263,7 +274,8 @@ DEVINL float moe_gated_act(float g, float u, int act, float limit) {
 }
 
 // hmid[r, f] = act(gate_e[f] . x, up_e[f] . x);  gate_up [E, 2F, W]; a null w
-// leaves the input unscaled (x = h[t])
+// leaves the input unscaled (x = h[t]). Ungated activations: hmid[r, f] =
+// act(up_e[f] . x) with gate_up [E, F, W].
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gate_up_gemv_kernel(
     T* __restrict__ hmid, const T* __restrict__ h, const int* __restrict__ idx,
@@ -278,10 +290,15 @@ __global__ __launch_bounds__(256) void moe_gate_up_gemv_kernel(
     xs[i] = w ? to_f32(from_f32<T>(wr * to_f32(h[t * W + i]))) : to_f32(h[t * W + i]);
   __syncthreads();
   const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-  const T* ge = gate_up + (long)e * 2 * F * W;
+  const bool gated = act < kMoeActGeluErf;
+  const T* ge = gate_up + (long)e * (gated ? 2 : 1) * F * W;
   const int f0 = (blockIdx.x * 4 + wv) * kMoeRowsPerWave;
   for (int f = f0; f < min(F, f0 + kMoeRowsPerWave); ++f) {
     const float g = to_f32(from_f32<T>(wave_dot(ge + (long)f * W, xs, W, lane)));
+    if (!gated) {
+      if (lane == 0) hmid[r * F + f] = from_f32<T>(moe_plain_act(g, act));
+      continue;
+    }
     const float u = to_f32(from_f32<T>(wave_dot(ge + (long)(F + f) * W, xs, W, lane)));
     if (lane == 0) hmid[r * F + f] = from_f32<T>(moe_gated_act(g, u, act, limit));
   }

@@ -779,10 +779,12 @@ def test_router_with_correction(target, E, top, T):
 
 @pytest.mark.parametrize("target", DEVICES)
 @pytest.mark.parametrize("W,F,E,ident,top,T", [(48, 24, 5, 2, 3, 9), (40, 20, 3, 0, 2, 3),
+                                               (48, 24, 5, 2, 3, 4), (56, 33, 6, 3, 2, 1),
                                                (36, 10, 3, 3, 3, 130), (64, 32, 8, 2, 2, 700)])
 def test_expert_mixture_with_identity_experts(target, W, F, E, ident, top, T):
     """Ungated GELU experts and identity experts through every form of the
-    expert op (sorted, and the batched form decode graphs use)."""
+    expert op (sorted, the batched form decode graphs use, and for few rows
+    the matrix-vector kernels that read only the chosen experts)."""
     device, dtype = dev_dtype(target)
     g = torch.Generator().manual_seed(W + T)
     h = torch.randn(T, W, generator=g).to(dtype)
