@@ -276,6 +276,7 @@ void paged_attn_prefill(at::Tensor out, at::Tensor q, const std::optional<at::Te
                                   q.stride(0) % 8 == 0 && !gate.has_value()),
               "rows that share a position run on the matrix-core kernel only");
   if (q.scalar_type() == at::kBFloat16 && (!force_valu || pos_stride == 0) && a.D % 8 == 0 && a.D <= 256 &&
+      a.DV <= 256 &&   // 16 channel tiles of 16 per wave; wider values run on the fp32 ALUs
       q.stride(0) % 8 == 0 && reinterpret_cast<uintptr_t>(q.data_ptr()) % 16 == 0) {
     const int ksn = (a.D + 31) / 32, dtn = (a.DV + 15) / 16;
     // rows that share a position (single tokens): a sequence is one

@@ -607,6 +607,16 @@ def test_sink_and_score_cap(target, decode):
 
 
 @pytest.mark.parametrize("target", DEVICES)
+@pytest.mark.parametrize("decode", [False, True], ids=["portion", "single"])
+def test_values_wider_than_the_matrix_core_tiles(target, decode):
+    device, dtype = dev_dtype(target)
+    tol = 2e-2 if dtype == torch.bfloat16 else 1e-5
+    got = _needle(device, dtype, 70, 100, decode, 40, 3, sink=1.0, DV=320)
+    want = _needle_weight(70, 100, 40, 3, sink=1.0)
+    assert abs(got - want) < tol * want
+
+
+@pytest.mark.parametrize("target", DEVICES)
 def test_sink_is_per_head(target):
     device, dtype = dev_dtype(target)
     H, D = 3, 8
